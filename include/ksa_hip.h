@@ -1,0 +1,114 @@
+/* libksa_hip.so — C ABI of the MI355X (gfx950) Summary-Attention kernels.
+ *
+ * The reference (Kuaishou-OneRec/KSA) has no C/FFI boundary on these paths: its two
+ * boundaries are Python call sites.  Each entry point below names the Python-level
+ * reference interface it stands behind ("whl-sa" = summary_attn-0.3.0 wheel,
+ * "whl-fa" = flash_attn_cute-0.1.0 wheel, "HF" =
+ * examples/pretrain/hf_template/modeling_qwen3sa.py).
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer owned by the caller unless stated otherwise;
+ *     the library never allocates, frees or synchronises;
+ *   - `stream` is a hipStream_t passed as void* (0 = the null stream);
+ *   - 16-bit tensors are described by element strides; pointers must be 16-byte
+ *     aligned and strides multiples of 8 elements, the innermost (head_dim) stride is 1;
+ *   - dtype: 0 = bf16, 1 = fp16; head_dim 64 or 128;
+ *   - return value 0 = launched, negative = rejected before any launch
+ *     (see ksa_error_string).
+ */
+#ifndef KSA_HIP_H
+#define KSA_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define KSA_OK 0
+#define KSA_ERR_INVALID (-1)
+#define KSA_ERR_NULL (-2)
+#define KSA_ERR_UNSUPPORTED (-3)
+#define KSA_ERR_WORKSPACE (-4)
+#define KSA_ERR_LAUNCH (-5)
+#define KSA_ERR_ALIGN (-6)
+
+#define KSA_DTYPE_BF16 0
+#define KSA_DTYPE_F16 1
+
+int ksa_version(void);
+const char* ksa_error_string(int code);
+int ksa_device_cu_count(void);
+
+/* Block-sparsity index.
+ * Replaces whl-fa:flash_attn/cute/compute_block_sparsity.py:276-375 (compute_block_sparsity)
+ * as called from whl-sa:summary_attn/interface.py:36-68 with (tile_m, tile_n, 1, 1, Sq, Sk)
+ * and the predicate of whl-sa:summary_attn/mask.py chosen by (P > 0, skip_old).
+ * P must equal Sk - Sq.  Outputs (int32, fully written, zero padded, ascending n):
+ *   mask_cnt[M], mask_idx[M*N], full_cnt[M], full_idx[M*N],
+ *   M = ceil(Sq/tile_m), N = ceil(Sk/tile_n). */
+int ksa_block_index(int Sq, int Sk, int C, int S, int W, int P, int skip_old, int tile_m,
+                    int tile_n, int32_t* mask_cnt, int32_t* mask_idx, int32_t* full_cnt,
+                    int32_t* full_idx, void* stream);
+
+/* Prefill forward.
+ * Replaces whl-sa:summary_attn/interface.py:271-289 (summary_attn_func) ->
+ * :70-91 (SummaryAttnFunc.forward) -> whl-fa:flash_attn/cute/interface.py:85-534
+ * (_flash_attn_fwd with mask_mod + block_sparse_tensors, tiles 128 x 64).
+ *   q   [batch, Sq, Hq,  D]   strides {batch, row, head}
+ *   k,v [batch, Sq, Hkv, D]   in-line keys / values
+ *   kprefix, vprefix: the P summary rows as separate tensors [batch, P, Hkv, D], or NULL:
+ *       then prefix row j is read in place from in-line row (j/S)*(C+S) + C + j%S
+ *       (what `k[:, summary_pos]` gathers when summary_pos is the periodic pattern).
+ *   out [batch, Sq, Hq, D]; lse fp32 [batch, Hq, Sq] (natural log) or NULL.
+ *   mask_cnt .. full_idx: output of ksa_block_index(Sq, Sq+P, ..., 128, 64), idx_stride = N.
+ *   scale: soft-max scale (the reference uses head_dim^-0.5). */
+int ksa_prefill_fwd(const void* q, const void* k, const void* v, const void* kprefix,
+                    const void* vprefix, void* out, float* lse, int batch, int Sq, int Hq, int Hkv,
+                    int D, int dtype, const int64_t* q_strides, const int64_t* k_strides,
+                    const int64_t* v_strides, const int64_t* kprefix_strides,
+                    const int64_t* vprefix_strides, const int64_t* out_strides, int C, int S, int W,
+                    int P, int skip_old, const int32_t* mask_cnt, const int32_t* mask_idx,
+                    const int32_t* full_cnt, const int32_t* full_idx, int idx_stride, float scale,
+                    void* stream);
+
+/* Decode attention over the ring-buffer slice.
+ * Replaces HF:591-612 (_sdpa_attention_forward, incl. repeat_kv :557-566) applied to the
+ * slice of HF:402-434 (Qwen3RingBufferCache.get_attention_kv).
+ *   q      [batch, Hq, Q, D]      strides {batch, head, query}
+ *   kcache [batch, Hkv, rows, D]  strides {batch, head, row}   (same for vcache)
+ *   out    [batch, Q, Hq, D]      strides {batch, query, head}
+ *   rows attended for sequence b: [start[b], end[b]) if start/end (device int32[batch])
+ *   are given, else [start0, end0) for every sequence.  No mask, no causality.
+ *   nsplit >= 1 splits of the row range; nsplit > 1 needs a workspace of
+ *   ksa_decode_workspace_bytes(...) bytes (fp32 partials). */
+size_t ksa_decode_workspace_bytes(int batch, int Hq, int Hkv, int Q, int D, int nsplit);
+int ksa_decode_auto_splits(int batch, int Hkv, int max_rows);
+int ksa_decode_fwd(const void* q, const void* kcache, const void* vcache, void* out,
+                   const int32_t* start, const int32_t* end, int start0, int end0, int batch,
+                   int Hq, int Hkv, int Q, int D, int dtype, const int64_t* q_strides,
+                   const int64_t* k_strides, const int64_t* v_strides, const int64_t* out_strides,
+                   float scale, int nsplit, void* workspace, size_t workspace_bytes, void* stream);
+
+/* Cache row mover.
+ * Replaces the Tensor.copy_ sequences of HF:306-336 (update_text), HF:340-398
+ * (update_summary), HF:209-302 (reorganize_after_prefill) and the boolean gather of
+ * whl-sa:summary_attn/interface.py:276-278.
+ * For every (sequence, head): dst row (dst_start + i) <- src row (src_index ? src_index[i]
+ * : src_start + i), i < nrows; dst_start_seq (device int32[batch]) overrides dst_start
+ * per sequence.  Tensors are [batch, heads, rows, D] by strides {batch, head, row}. */
+int ksa_copy_rows(const void* src, void* dst, const int32_t* src_index,
+                  const int32_t* dst_start_seq, int src_start, int dst_start, int nrows, int batch,
+                  int heads, int D, const int64_t* src_strides, const int64_t* dst_strides,
+                  void* stream);
+
+/* Host-side diagnostic: number of key columns in [a, b) visible to query row q under the
+ * closed-form rule the kernels use (no GPU involved). */
+long long ksa_debug_count_visible(long long q, long long a, long long b, int C, int S, int W,
+                                  int P, int skip_old, int Sq, int Sk);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KSA_HIP_H */

@@ -1,0 +1,69 @@
+"""ctypes binding of libksa_hip.so.  There is no fallback: if the library is missing
+or does not load, every operator of this package raises."""
+from __future__ import annotations
+
+import ctypes
+import os
+
+import torch  # noqa: F401  (must be imported first so that its HIP runtime is the one in the process)
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libksa_hip.so")
+_lib = None
+
+_i32p = ctypes.POINTER(ctypes.c_int32)
+_i64p = ctypes.POINTER(ctypes.c_int64)
+_vp = ctypes.c_void_p
+_int = ctypes.c_int
+
+_SIGNATURES = {
+    "ksa_version": (_int, []),
+    "ksa_error_string": (ctypes.c_char_p, [_int]),
+    "ksa_device_cu_count": (_int, []),
+    "ksa_block_index": (_int, [_int] * 9 + [_vp] * 4 + [_vp]),
+    "ksa_prefill_fwd": (_int, [_vp] * 7 + [_int] * 6 + [_i64p] * 6 + [_int] * 5 + [_vp] * 4
+                        + [_int, ctypes.c_float, _vp]),
+    "ksa_decode_workspace_bytes": (ctypes.c_size_t, [_int] * 6),
+    "ksa_decode_auto_splits": (_int, [_int] * 3),
+    "ksa_decode_fwd": (_int, [_vp] * 6 + [_int] * 8 + [_i64p] * 4
+                       + [ctypes.c_float, _int, _vp, ctypes.c_size_t, _vp]),
+    "ksa_copy_rows": (_int, [_vp] * 4 + [_int] * 6 + [_i64p] * 2 + [_vp]),
+    "ksa_debug_count_visible": (ctypes.c_longlong, [ctypes.c_longlong] * 3 + [_int] * 7),
+}
+
+EXPORTS = tuple(_SIGNATURES)
+
+
+class KsaError(RuntimeError):
+    pass
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise KsaError(
+                f"{LIB_PATH} is missing: build it with `python -m ksa_amd.build` "
+                "(hipcc, gfx950); ksa_amd has no other execution path")
+        L = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in _SIGNATURES.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = L
+    return _lib
+
+
+def check(code: int, what: str):
+    if code != 0:
+        msg = lib().ksa_error_string(code).decode()
+        raise KsaError(f"{what}: {msg} (code {code})")
+
+
+def strides3(t, dims):
+    """int64[3] of element strides of tensor `t` along the three named dims."""
+    return (ctypes.c_int64 * 3)(*[t.stride(d) for d in dims])
+
+
+def stream_ptr(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream

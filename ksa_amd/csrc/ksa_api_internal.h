@@ -1,0 +1,21 @@
+// Internal helpers shared by the translation units of libksa_hip.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+// status codes returned by every extern "C" entry point (0 = success)
+enum {
+    KSA_OK = 0,
+    KSA_ERR_INVALID = -1,      // a size / flag argument is out of range
+    KSA_ERR_NULL = -2,         // a required pointer is null
+    KSA_ERR_UNSUPPORTED = -3,  // dtype / head_dim not compiled in
+    KSA_ERR_WORKSPACE = -4,    // workspace too small
+    KSA_ERR_LAUNCH = -5,       // the HIP runtime refused the launch
+    KSA_ERR_ALIGN = -6,        // pointer or stride not 16-byte aligned
+};
+
+enum { KSA_DTYPE_BF16 = 0, KSA_DTYPE_F16 = 1 };
+
+static inline int ksa_check_launch() {
+    return hipGetLastError() == hipSuccess ? KSA_OK : KSA_ERR_LAUNCH;
+}

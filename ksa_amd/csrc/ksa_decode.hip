@@ -1,0 +1,373 @@
+// Decode attention over the contiguous ring-buffer KV slice for gfx950.
+//
+// Replaces the reference's decode attention function
+//   examples/pretrain/hf_template/modeling_qwen3sa.py:591-612 (_sdpa_attention_forward)
+//   examples/pretrain/hf_template/modeling_qwen3sa.py:557-566 (repeat_kv)
+// i.e. softmax(q K^T * scale) V without any mask over rows [start_b, end_b) of the
+// cache slice returned by Qwen3RingBufferCache.get_attention_kv (:402-434).  The
+// reference materialises g copies of K and V per step; here every K/V row is read
+// from HBM exactly once per kv head and shared by the g query heads (and by all
+// query tokens of a chunk-boundary step) as columns of one MFMA tile.
+//
+// Split-K: a workgroup owns (sequence, kv head, split); its 4 waves stream disjoint
+// 32-row tiles with private LDS staging (no workgroup barrier in the loop) and keep
+// private (max, sum, O^T) state that is merged across the waves through LDS at the
+// end; with more than one split the un-normalised partials go to a workspace and a
+// second kernel merges them.
+#include <hip/hip_runtime.h>
+#include <math.h>
+
+#include "ksa_api_internal.h"
+#include "ksa_tile.h"
+
+namespace {
+
+struct DecodeParams {
+    const uint16_t* q;
+    const uint16_t* k;
+    const uint16_t* v;
+    uint16_t* out;
+    const int32_t* start;  // per sequence or null
+    const int32_t* end;
+    int start0, end0;
+    int Hq, Hkv, g, Q;
+    int ncols;   // Q * g columns per kv head
+    int nsplit;
+    int64_t q_bs, q_hs, q_qs;   // element strides of q [B,Hq,Q,D]
+    int64_t k_bs, k_hs, k_rs;   // cache [B,Hkv,rows,D]
+    int64_t v_bs, v_hs, v_rs;
+    int64_t o_bs, o_qs, o_hs;   // out [B,Q,Hq,D]
+    float* ws_o;   // [B,Hkv,nsplit,ncols_pad,D] un-normalised partial outputs
+    float* ws_ml;  // [B,Hkv,nsplit,ncols_pad,2]  (max in log2 units, sum)
+    int ncols_pad;
+    float scale_log2;
+};
+
+constexpr int kThreads = 256;
+constexpr int kWaves = 4;
+constexpr int kRows = 32;  // key rows per wave tile
+
+template <typename T, int D>
+__global__ __launch_bounds__(kThreads, 2) void ksa_decode_kernel(const DecodeParams p) {
+    using Ops = KsaOps<T>;
+    constexpr int KS = D / 16;
+    constexpr int DB = D / 32;
+    constexpr int KROW = D + 8;
+    constexpr int VROW = kRows + 8;
+    constexpr int CPR = D / 8;
+    constexpr int KLD = (kRows * CPR) / 64;          // K loads per lane
+    constexpr int VUNITS = (kRows / 4) * CPR;
+    constexpr int VLD = (VUNITS + 63) / 64;
+    constexpr int kStage = kRows * KROW + D * VROW;  // elements of one wave's staging area
+    constexpr int kMergeFloats = kWaves * 32 * (D + 2);
+    constexpr int kSmemBytes = (kWaves * kStage * 2 > kMergeFloats * 4) ? kWaves * kStage * 2
+                                                                        : kMergeFloats * 4;
+    __shared__ __attribute__((aligned(16))) unsigned char smem[kSmemBytes];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int lq = lane & 31;
+    const int lh = lane >> 5;
+
+    const int split = blockIdx.x;
+    const int colblk = blockIdx.y / p.Hkv;
+    const int kvh = blockIdx.y % p.Hkv;
+    const int bz = blockIdx.z;
+
+    uint16_t* Kw = reinterpret_cast<uint16_t*>(smem) + wave * kStage;
+    uint16_t* Vw = Kw + kRows * KROW;
+
+    const int r_begin = p.start ? p.start[bz] : p.start0;
+    const int r_end = p.end ? p.end[bz] : p.end0;
+    const int L = max(r_end - r_begin, 0);
+    // rows per split: a multiple of the 128 rows the four waves cover per round
+    const int per = ((L + p.nsplit - 1) / p.nsplit + kWaves * kRows - 1) / (kWaves * kRows) *
+                    (kWaves * kRows);
+    const int s0 = r_begin + split * per;
+    const int s1 = min(r_end, s0 + per);
+
+    // column (query token qi, head gi of the group) owned by this lane
+    const int col = colblk * 32 + lq;
+    const bool col_ok = col < p.ncols;
+    const int qi = col_ok ? col / p.g : 0;
+    const int gi = col_ok ? col % p.g : 0;
+    const int head = kvh * p.g + gi;
+
+    u32x4 qf[KS];
+    {
+        const uint16_t* qp = p.q + bz * p.q_bs + head * p.q_hs + qi * p.q_qs + 8 * lh;
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+            u32x4 z = {0u, 0u, 0u, 0u};
+            qf[s] = col_ok ? *reinterpret_cast<const u32x4*>(qp + 16 * s) : z;
+        }
+    }
+
+    const uint16_t* kbase = p.k + bz * p.k_bs + kvh * p.k_hs;
+    const uint16_t* vbase = p.v + bz * p.v_bs + kvh * p.v_hs;
+    const int last_row = max(r_end - 1, r_begin);
+
+    u32x4 kreg[KLD];
+    u32x4 vreg[VLD][4];
+
+    auto load_tile = [&](int row0) {
+#pragma unroll
+        for (int i = 0; i < KLD; ++i) {
+            const int u = lane + 64 * i;
+            const int row = min(row0 + u / CPR, last_row);
+            kreg[i] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)row * p.k_rs + 8 * (u % CPR));
+        }
+#pragma unroll
+        for (int i = 0; i < VLD; ++i) {
+            const int u = lane + 64 * i;
+            if (u < VUNITS) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int row = min(row0 + 4 * (u / CPR) + r, last_row);
+                    vreg[i][r] =
+                        *reinterpret_cast<const u32x4*>(vbase + (int64_t)row * p.v_rs + 8 * (u % CPR));
+                }
+            }
+        }
+    };
+
+    floatx16 oacc[DB];
+#pragma unroll
+    for (int b = 0; b < DB; ++b)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) oacc[b][i] = 0.f;
+    float m_run = -INFINITY;  // in raw score units
+    float l_run = 0.f;
+    const float c2 = p.scale_log2;
+
+    int row0 = s0 + wave * kRows;
+    if (row0 < s1) load_tile(row0);
+
+    for (; row0 < s1; row0 += kWaves * kRows) {
+        ksa_wave_lds_fence();
+#pragma unroll
+        for (int i = 0; i < KLD; ++i) {
+            const int u = lane + 64 * i;
+            *reinterpret_cast<u32x4*>(Kw + (u / CPR) * KROW + 8 * (u % CPR)) = kreg[i];
+        }
+#pragma unroll
+        for (int i = 0; i < VLD; ++i) {
+            const int u = lane + 64 * i;
+            if (u < VUNITS) ksa_store_vt<VROW>(Vw, 8 * (u % CPR), ksa_vt_pos(u / CPR), vreg[i]);
+        }
+        ksa_wave_lds_fence();
+        const int next = row0 + kWaves * kRows;
+        if (next < s1) load_tile(next);
+
+        floatx16 sacc;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sacc[i] = 0.f;
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+            const u32x4 a = *reinterpret_cast<const u32x4*>(Kw + lq * KROW + 16 * s + 8 * lh);
+            sacc = Ops::mfma(a, qf[s], sacc);
+        }
+        if (row0 + kRows > s1) {  // tail tile: rows past the slice end do not exist
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int r = row0 + 8 * (i / 4) + 4 * lh + (i % 4);
+                if (r >= s1) sacc[i] = -INFINITY;
+            }
+        }
+        float mloc = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) mloc = fmaxf(mloc, sacc[i]);
+        mloc = fmaxf(mloc, ksa_xor32(mloc));
+        const float m_new = fmaxf(m_run, mloc);  // finite: every tile has >= 1 real row
+        const float alpha = ksa_exp2((m_run - m_new) * c2);
+        const float mc = m_new * c2;
+        m_run = m_new;
+        float rowsum = 0.f;
+        u32x4 pf[2];
+#pragma unroll
+        for (int i = 0; i < 16; i += 2) {
+            const float p0 = ksa_exp2(fmaf(sacc[i], c2, -mc));
+            const float p1 = ksa_exp2(fmaf(sacc[i + 1], c2, -mc));
+            rowsum += p0 + p1;
+            pf[i / 8][(i % 8) / 2] = Ops::pack2(p0, p1);
+        }
+        l_run = l_run * alpha + rowsum;
+        if (__any(alpha != 1.f)) {
+#pragma unroll
+            for (int b = 0; b < DB; ++b)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) oacc[b][i] *= alpha;
+        }
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int b = 0; b < DB; ++b) {
+                const u32x4 a =
+                    *reinterpret_cast<const u32x4*>(Vw + (b * 32 + lq) * VROW + 16 * ks + 8 * lh);
+                oacc[b] = Ops::mfma(a, pf[ks], oacc[b]);
+            }
+    }
+
+    // ---- merge the four waves through LDS ----
+    l_run += ksa_xor32(l_run);
+    __syncthreads();  // staging areas are dead from here on
+    float* mg = reinterpret_cast<float*>(smem);  // [wave][col 32][D + 2]
+    {
+        float* row = mg + (wave * 32 + lq) * (D + 2);
+#pragma unroll
+        for (int b = 0; b < DB; ++b)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) row[32 * b + 8 * (i / 4) + 4 * lh + (i % 4)] = oacc[b][i];
+        if (lh == 0) {
+            row[D] = m_run * c2;  // log2 units; -inf if this wave saw no row
+            row[D + 1] = l_run;
+        }
+    }
+    __syncthreads();
+    const int ncol_here = min(32, p.ncols - colblk * 32);
+    for (int e = tid; e < ncol_here * D; e += kThreads) {
+        const int c = e / D, d = e % D;
+        float mx = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) mx = fmaxf(mx, mg[(w * 32 + c) * (D + 2) + D]);
+        float acc = 0.f, l = 0.f;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+            const float* row = mg + (w * 32 + c) * (D + 2);
+            const float f = (row[D] == -INFINITY) ? 0.f : ksa_exp2(row[D] - mx);
+            acc += row[d] * f;
+            l += row[D + 1] * f;
+        }
+        const int cg = colblk * 32 + c;
+        if (p.nsplit == 1) {
+            const int oq = cg / p.g, og = cg % p.g;
+            const float val = l > 0.f ? acc / l : 0.f;
+            uint16_t* op = p.out + bz * p.o_bs + oq * p.o_qs + (kvh * p.g + og) * p.o_hs + d;
+            const uint32_t pk = Ops::pack2(val, 0.f);
+            *op = (uint16_t)(pk & 0xffffu);
+        } else {
+            const int64_t slot = (((int64_t)bz * p.Hkv + kvh) * p.nsplit + split) * p.ncols_pad + cg;
+            p.ws_o[slot * D + d] = acc;
+            if (d == 0) {
+                p.ws_ml[slot * 2] = mx;
+                p.ws_ml[slot * 2 + 1] = l;
+            }
+        }
+    }
+}
+
+// second stage: merge the splits of one (sequence, kv head, column)
+template <typename T, int D>
+__global__ __launch_bounds__(D) void ksa_decode_merge_kernel(const DecodeParams p) {
+    using Ops = KsaOps<T>;
+    const int cg = blockIdx.x;
+    const int kvh = blockIdx.y;
+    const int bz = blockIdx.z;
+    const int d = threadIdx.x;
+    const int64_t base = (((int64_t)bz * p.Hkv + kvh) * p.nsplit) * p.ncols_pad + cg;
+    float mx = -INFINITY;
+    for (int s = 0; s < p.nsplit; ++s) mx = fmaxf(mx, p.ws_ml[(base + (int64_t)s * p.ncols_pad) * 2]);
+    float acc = 0.f, l = 0.f;
+    for (int s = 0; s < p.nsplit; ++s) {
+        const int64_t slot = base + (int64_t)s * p.ncols_pad;
+        const float m = p.ws_ml[slot * 2];
+        const float f = (m == -INFINITY) ? 0.f : ksa_exp2(m - mx);
+        acc += p.ws_o[slot * D + d] * f;
+        l += p.ws_ml[slot * 2 + 1] * f;
+    }
+    const int oq = cg / p.g, og = cg % p.g;
+    const float val = l > 0.f ? acc / l : 0.f;
+    uint16_t* op = p.out + bz * p.o_bs + oq * p.o_qs + (kvh * p.g + og) * p.o_hs + d;
+    *op = (uint16_t)(Ops::pack2(val, 0.f) & 0xffffu);
+}
+
+template <typename T, int D>
+int launch(const DecodeParams& p, int batch, hipStream_t stream) {
+    const int colblks = (p.ncols + 31) / 32;
+    dim3 grid(p.nsplit, p.Hkv * colblks, batch);
+    hipLaunchKernelGGL((ksa_decode_kernel<T, D>), grid, dim3(kThreads), 0, stream, p);
+    if (p.nsplit > 1) {
+        dim3 g2(p.ncols, p.Hkv, batch);
+        hipLaunchKernelGGL((ksa_decode_merge_kernel<T, D>), g2, dim3(D), 0, stream, p);
+    }
+    return ksa_check_launch();
+}
+
+int pad_cols(int ncols) { return (ncols + 31) / 32 * 32; }
+
+}  // namespace
+
+extern "C" size_t ksa_decode_workspace_bytes(int batch, int Hq, int Hkv, int Q, int D, int nsplit) {
+    if (nsplit <= 1 || batch <= 0 || Hkv <= 0 || Hq % Hkv != 0) return 0;
+    const size_t cols = (size_t)pad_cols(Q * (Hq / Hkv));
+    return (size_t)batch * Hkv * nsplit * cols * (D + 2) * sizeof(float);
+}
+
+// Heuristic number of splits: enough workgroups to cover the 256 CUs a few times
+// over, but never splits shorter than 256 rows.
+extern "C" int ksa_decode_auto_splits(int batch, int Hkv, int max_rows) {
+    if (batch <= 0 || Hkv <= 0 || max_rows <= 0) return 1;
+    const int units = batch * Hkv;
+    int n = (1024 + units - 1) / units;
+    const int cap = max_rows / 256 > 1 ? max_rows / 256 : 1;
+    if (n > cap) n = cap;
+    if (n > 64) n = 64;
+    return n < 1 ? 1 : n;
+}
+
+extern "C" int ksa_decode_fwd(const void* q, const void* kcache, const void* vcache, void* out,
+                              const int32_t* start, const int32_t* end, int start0, int end0,
+                              int batch, int Hq, int Hkv, int Q, int D, int dtype,
+                              const int64_t* q_strides, const int64_t* k_strides,
+                              const int64_t* v_strides, const int64_t* out_strides, float scale,
+                              int nsplit, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!q || !kcache || !vcache || !out || !q_strides || !k_strides || !v_strides || !out_strides)
+        return KSA_ERR_NULL;
+    if ((start == nullptr) != (end == nullptr)) return KSA_ERR_NULL;
+    if (batch <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || Q <= 0 || nsplit < 1) return KSA_ERR_INVALID;
+    if (!start && (start0 < 0 || end0 <= start0)) return KSA_ERR_INVALID;
+    if (dtype != KSA_DTYPE_BF16 && dtype != KSA_DTYPE_F16) return KSA_ERR_UNSUPPORTED;
+    if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(kcache) |
+         reinterpret_cast<uintptr_t>(vcache)) & 15)
+        return KSA_ERR_ALIGN;
+    for (int i = 0; i < 3; ++i)
+        if ((q_strides[i] % 8) || (k_strides[i] % 8) || (v_strides[i] % 8)) return KSA_ERR_ALIGN;
+
+    DecodeParams p{};
+    p.q = (const uint16_t*)q;
+    p.k = (const uint16_t*)kcache;
+    p.v = (const uint16_t*)vcache;
+    p.out = (uint16_t*)out;
+    p.start = start;
+    p.end = end;
+    p.start0 = start0;
+    p.end0 = end0;
+    p.Hq = Hq;
+    p.Hkv = Hkv;
+    p.g = Hq / Hkv;
+    p.Q = Q;
+    p.ncols = Q * p.g;
+    p.ncols_pad = pad_cols(p.ncols);
+    p.nsplit = nsplit;
+    p.q_bs = q_strides[0], p.q_hs = q_strides[1], p.q_qs = q_strides[2];
+    p.k_bs = k_strides[0], p.k_hs = k_strides[1], p.k_rs = k_strides[2];
+    p.v_bs = v_strides[0], p.v_hs = v_strides[1], p.v_rs = v_strides[2];
+    p.o_bs = out_strides[0], p.o_qs = out_strides[1], p.o_hs = out_strides[2];
+    p.scale_log2 = scale * 1.4426950408889634f;
+    if (nsplit > 1) {
+        const size_t need = ksa_decode_workspace_bytes(batch, Hq, Hkv, Q, D, nsplit);
+        if (!workspace || workspace_bytes < need) return KSA_ERR_WORKSPACE;
+        p.ws_o = (float*)workspace;
+        p.ws_ml = p.ws_o + (size_t)batch * Hkv * nsplit * p.ncols_pad * D;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == KSA_DTYPE_BF16) {
+        if (D == 128) return launch<KsaBf16, 128>(p, batch, st);
+        if (D == 64) return launch<KsaBf16, 64>(p, batch, st);
+    } else {
+        if (D == 128) return launch<KsaF16, 128>(p, batch, st);
+        if (D == 64) return launch<KsaF16, 64>(p, batch, st);
+    }
+    return KSA_ERR_UNSUPPORTED;
+}

@@ -1,0 +1,100 @@
+"""Decode attention over the contiguous ring-buffer KV slice on MI355X.
+
+`decode_attention_forward` has the signature of the reference's `_decode_attn_fn`
+(examples/pretrain/hf_template/modeling_qwen3sa.py:591-612 `_sdpa_attention_forward`,
+selected at :643-646 and called at :820-830, :844-870): un-masked, non-causal
+soft-max attention of `query [b, Hq, q_len, D]` over `key/value [b, Hkv, L, D]`
+(strided views of the cache), GQA by `module.num_key_value_groups`, returning
+`(attn_output [b, q_len, Hq, D], None)`.  `ksa_decode` is the lower-level form that
+takes the whole cache tensor and per-sequence row ranges, which the reference cannot
+express (its cache counters are shared by the batch, :753-754).
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+
+_DTYPES = {torch.bfloat16: 0, torch.float16: 1}
+
+
+@torch.library.custom_op("ksa_amd::decode_fwd", mutates_args=())
+def _decode_fwd(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
+                start: Optional[torch.Tensor], end: Optional[torch.Tensor], start0: int, end0: int,
+                scale: float, nsplit: int) -> torch.Tensor:
+    b, Hq, Q, D = q.shape
+    Hkv = kcache.shape[1]
+    lib = _lib.lib()
+    out = torch.empty((b, Q, Hq, D), dtype=q.dtype, device=q.device)
+    ws = None
+    ws_bytes = 0
+    if nsplit > 1:
+        ws_bytes = lib.ksa_decode_workspace_bytes(b, Hq, Hkv, Q, D, nsplit)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+    with torch.cuda.device(q.device):
+        rc = lib.ksa_decode_fwd(
+            q.data_ptr(), kcache.data_ptr(), vcache.data_ptr(), out.data_ptr(),
+            start.data_ptr() if start is not None else None,
+            end.data_ptr() if end is not None else None, start0, end0,
+            b, Hq, Hkv, Q, D, _DTYPES[q.dtype],
+            _lib.strides3(q, (0, 1, 2)), _lib.strides3(kcache, (0, 1, 2)),
+            _lib.strides3(vcache, (0, 1, 2)), _lib.strides3(out, (0, 1, 2)),
+            float(scale), nsplit, ws.data_ptr() if ws is not None else None, ws_bytes,
+            _lib.stream_ptr(q.device))
+    _lib.check(rc, "ksa_decode_fwd")
+    return out
+
+
+@_decode_fwd.register_fake
+def _(q, kcache, vcache, start, end, start0, end0, scale, nsplit):
+    b, Hq, Q, D = q.shape
+    return q.new_empty((b, Q, Hq, D))
+
+
+def ksa_decode(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
+               start=None, end=None, scale: Optional[float] = None,
+               nsplit: Optional[int] = None) -> torch.Tensor:
+    """q [b, Hq, Q, D]; kcache/vcache [b, Hkv, rows, D] (any batch/head/row strides);
+    rows [start, end) are attended: ints for every sequence, or int32 device tensors [b]
+    per sequence; default is the whole row axis.  Returns [b, Q, Hq, D]."""
+    assert q.is_cuda and kcache.is_cuda and vcache.is_cuda, "inputs must be on a GPU"
+    assert q.dtype in _DTYPES and q.dtype == kcache.dtype == vcache.dtype, "inputs must share a 16-bit float dtype"
+    assert q.dim() == 4 and kcache.dim() == 4 and kcache.shape == vcache.shape
+    b, Hq, Q, D = q.shape
+    assert kcache.shape[0] == b and kcache.shape[3] == D and Hq % kcache.shape[1] == 0
+    if q.stride(-1) != 1:
+        q = q.contiguous()
+    assert kcache.stride(-1) == 1 and vcache.stride(-1) == 1, "cache rows must be contiguous"
+    rows = kcache.shape[2]
+    t_start = t_end = None
+    s0, e0 = 0, rows
+    if isinstance(start, torch.Tensor) or isinstance(end, torch.Tensor):
+        t_start = torch.as_tensor(start if start is not None else 0, device=q.device).to(torch.int32).expand(b).contiguous()
+        t_end = torch.as_tensor(end if end is not None else rows, device=q.device).to(torch.int32).expand(b).contiguous()
+        max_rows = rows
+    else:
+        s0 = 0 if start is None else int(start)
+        e0 = rows if end is None else int(end)
+        assert 0 <= s0 < e0 <= rows, "row range out of bounds"
+        max_rows = e0 - s0
+    if scale is None:
+        scale = float(D) ** -0.5
+    if nsplit is None:
+        nsplit = _lib.lib().ksa_decode_auto_splits(b, kcache.shape[1], max_rows)
+    return torch.ops.ksa_amd.decode_fwd(q, kcache, vcache, t_start, t_end, s0, e0, float(scale), int(nsplit))
+
+
+def decode_attention_forward(module, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
+                             attention_mask: Optional[torch.Tensor] = None,
+                             scaling: Optional[float] = None, dropout: float = 0.0,
+                             **kwargs) -> Tuple[torch.Tensor, None]:
+    """Drop-in for `Qwen3Attention._decode_attn_fn`.  `attention_mask` is ignored exactly
+    as the reference's SDPA variant ignores it (it passes attn_mask=None); dropout must be 0."""
+    if dropout:
+        raise NotImplementedError("decode attention is inference-only (dropout must be 0)")
+    g = query.shape[1] // key.shape[1]
+    mg = getattr(module, "num_key_value_groups", g)
+    assert mg == g, "module.num_key_value_groups does not match the tensor shapes"
+    return ksa_decode(query, key, value, scale=scaling), None

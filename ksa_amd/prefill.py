@@ -1,0 +1,207 @@
+"""Block-sparse Summary-Attention prefill forward on MI355X.
+
+Mirror of the reference's public prefill operator
+(summary_attn-0.3.0 wheel, summary_attn/interface.py:271-289 `summary_attn_func`;
+call sites: examples/pretrain/hf_template/modeling_qwen3sa.py:806-815 and
+muse/layers/summary_attention_func.py:67-73): same positional arguments, same
+keywords, same `(out, lse_or_None)` return.  The work is done by the HIP kernels of
+libksa_hip.so; there is no other execution path.
+"""
+from __future__ import annotations
+
+import ctypes
+import weakref
+from typing import Dict, Optional, Tuple
+
+import torch
+
+from . import _lib
+
+TILE_M = 128
+TILE_N = 64
+
+# (Sq, C, S, W, P, skip_old, device index) -> (mask_cnt, mask_idx, full_cnt, full_idx)
+# The reference keeps the same process-global cache keyed by shape parameters
+# (summary_attn/interface.py:26,46-68); the device is added to the key here because the
+# tensors live on one.
+SUMMARY_ATTN_CACHE: Dict[Tuple, Tuple[torch.Tensor, ...]] = {}
+
+_DTYPES = {torch.bfloat16: 0, torch.float16: 1}
+
+
+class BlockSparseIndex(tuple):
+    """(mask_block_cnt, mask_block_idx, full_block_cnt, full_block_idx) with the
+    reference's shapes [1,1,M] / [1,1,M,N] (flash_attn/cute/block_sparsity.py:17-34)."""
+
+    block_size = (TILE_M, TILE_N)
+
+
+def compute_block_sparsity(seqlen_q: int, seqlen_k: int, chunk_size: int, summary_num: int,
+                           sliding_chunk_num: int, skip_old_summary: bool = False,
+                           tile_m: int = TILE_M, tile_n: int = TILE_N,
+                           device=None) -> BlockSparseIndex:
+    """Builds the four int32 index tensors on the GPU (bit-exact with the reference's
+    BlockSparsityKernel, flash_attn/cute/compute_block_sparsity.py:189-274)."""
+    device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    if device.type != "cuda":
+        raise AssertionError("compute_block_sparsity runs on the GPU only")
+    M = -(-seqlen_q // tile_m)
+    N = -(-seqlen_k // tile_n)
+    with torch.cuda.device(device):
+        mc = torch.empty((1, 1, M), dtype=torch.int32, device=device)
+        fc = torch.empty((1, 1, M), dtype=torch.int32, device=device)
+        mi = torch.empty((1, 1, M, N), dtype=torch.int32, device=device)
+        fi = torch.empty((1, 1, M, N), dtype=torch.int32, device=device)
+        rc = _lib.lib().ksa_block_index(
+            seqlen_q, seqlen_k, chunk_size, summary_num, sliding_chunk_num, seqlen_k - seqlen_q,
+            int(bool(skip_old_summary)), tile_m, tile_n, mc.data_ptr(), mi.data_ptr(),
+            fc.data_ptr(), fi.data_ptr(), _lib.stream_ptr(device))
+    _lib.check(rc, "ksa_block_index")
+    return BlockSparseIndex((mc, mi, fc, fi))
+
+
+def _cached_index(Sq, C, S, W, P, skip_old, device) -> BlockSparseIndex:
+    key = (Sq, C, S, W, P, bool(skip_old), device.index)
+    idx = SUMMARY_ATTN_CACHE.get(key)
+    if idx is None:
+        idx = compute_block_sparsity(Sq, Sq + P, C, S, W, skip_old, device=device)
+        SUMMARY_ATTN_CACHE[key] = idx
+    return idx
+
+
+# summary_pos analysis is cached per tensor object (HF passes the same mask to every layer)
+# id(tensor) -> (weakref to it, version, (Sq, C, S), result)
+_POS_CACHE: Dict[int, tuple] = {}
+
+
+def _analyse_summary_pos(summary_pos: torch.Tensor, Sq: int, C: int, S: int):
+    """Returns (P, periodic, rows): P = number of summary rows; periodic = summary_pos
+    is exactly `(i % (C+S)) >= C` over whole blocks followed by text rows only, so that
+    prefix row j can be read in place at (j//S)*(C+S)+C+j%S; rows = int32 row indices of
+    the summary rows (only when not periodic)."""
+    hit = _POS_CACHE.get(id(summary_pos))
+    ver = summary_pos._version
+    if hit is not None and hit[0]() is summary_pos and hit[1] == ver and hit[2] == (Sq, C, S):
+        return hit[3]
+    if summary_pos.dtype != torch.bool or summary_pos.dim() != 1 or summary_pos.numel() != Sq:
+        raise AssertionError("summary_pos must be a bool tensor of shape [seqlen_q]")
+    B = C + S
+    i = torch.arange(Sq, device=summary_pos.device)
+    n_sum = summary_pos.sum()
+    n_full = n_sum // S
+    expected = ((i % B) >= C) & (i < n_full * B)
+    stats = torch.stack([n_sum, (summary_pos != expected).sum()]).tolist()  # one sync
+    P, mismatch = int(stats[0]), int(stats[1])
+    periodic = mismatch == 0 and P % S == 0
+    rows = None
+    if not periodic:
+        rows = torch.nonzero(summary_pos, as_tuple=False).flatten().to(torch.int32)
+    res = (P, periodic, rows)
+    if len(_POS_CACHE) > 64:
+        _POS_CACHE.clear()
+    _POS_CACHE[id(summary_pos)] = (weakref.ref(summary_pos), ver, (Sq, C, S), res)
+    return res
+
+
+def _check_inputs(q, k, v):
+    assert q.is_cuda and k.is_cuda and v.is_cuda, "inputs must be on a GPU"
+    assert q.dtype in _DTYPES, "inputs must be float16 or bfloat16"
+    assert q.dtype == k.dtype == v.dtype, "inputs must have the same dtype"
+    assert q.dim() == 4 and k.dim() == 4 and v.dim() == 4, "q/k/v must be [batch, seq, heads, head_dim]"
+    assert k.shape == v.shape, "k and v must have the same shape"
+    assert q.shape[0] == k.shape[0], "batch mismatch"
+    D = q.shape[-1]
+    assert k.shape[-1] == D, "head_dim mismatch"
+    assert D <= 256, "head dimension must be at most 256"
+    assert D % 8 == 0, "head dimension must be a multiple of 8"
+    assert q.shape[2] % k.shape[2] == 0, "num_heads must be divisible by num_heads_kv"
+
+
+def _lastdim_contig(t):
+    return t if t.stride(-1) == 1 else t.contiguous()
+
+
+@torch.library.custom_op("ksa_amd::summary_attn_fwd", mutates_args=())
+def _summary_attn_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                      kprefix: Optional[torch.Tensor], vprefix: Optional[torch.Tensor],
+                      mask_cnt: torch.Tensor, mask_idx: torch.Tensor, full_cnt: torch.Tensor,
+                      full_idx: torch.Tensor, C: int, S: int, W: int, P: int, skip_old: bool,
+                      scale: float, want_lse: bool) -> Tuple[torch.Tensor, torch.Tensor]:
+    b, Sq, Hq, D = q.shape
+    Hkv = k.shape[2]
+    out = torch.empty_like(q)
+    lse = torch.empty((b, Hq, Sq) if want_lse else (0,), dtype=torch.float32, device=q.device)
+    dims = (0, 1, 2)
+    null3 = ctypes.cast(None, ctypes.POINTER(ctypes.c_int64))
+    with torch.cuda.device(q.device):
+        rc = _lib.lib().ksa_prefill_fwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(),
+            kprefix.data_ptr() if kprefix is not None else None,
+            vprefix.data_ptr() if vprefix is not None else None,
+            out.data_ptr(), lse.data_ptr() if want_lse else None,
+            b, Sq, Hq, Hkv, D, _DTYPES[q.dtype],
+            _lib.strides3(q, dims), _lib.strides3(k, dims), _lib.strides3(v, dims),
+            _lib.strides3(kprefix, dims) if kprefix is not None else null3,
+            _lib.strides3(vprefix, dims) if vprefix is not None else null3,
+            _lib.strides3(out, dims), C, S, W, P, int(skip_old),
+            mask_cnt.data_ptr(), mask_idx.data_ptr(), full_cnt.data_ptr(), full_idx.data_ptr(),
+            mask_idx.shape[-1], float(scale), _lib.stream_ptr(q.device))
+    _lib.check(rc, "ksa_prefill_fwd")
+    return out, lse
+
+
+@_summary_attn_fwd.register_fake
+def _(q, k, v, kprefix, vprefix, mask_cnt, mask_idx, full_cnt, full_idx, C, S, W, P, skip_old,
+      scale, want_lse):
+    b, Sq, Hq, _ = q.shape
+    return torch.empty_like(q), q.new_empty((b, Hq, Sq) if want_lse else (0,), dtype=torch.float32)
+
+
+def summary_attn_func(q, k, v, chunk_size, summary_num, sliding_chunk_num,
+                      summary_pos: Optional[torch.Tensor] = None,
+                      skip_old_summary: bool = False, *, return_lse: bool = False,
+                      softmax_scale: Optional[float] = None):
+    """q [b, Sq, Hq, D]; k, v [b, Sq (+P), Hkv, D]; returns (out [b, Sq, Hq, D], lse or None).
+
+    With `summary_pos` (bool [Sq]) the summary rows of k/v form the key prefix, as
+    `torch.cat((k[:, summary_pos], k), dim=1)` does in the reference, but nothing is
+    concatenated: the kernel reads them where they are.  Without it, the first
+    `k.shape[1] - q.shape[1]` rows of k/v are taken as an already-built prefix.
+    Forward only: tensors that require grad under an enabled grad mode are rejected.
+    `return_lse` / `softmax_scale` are extensions (the reference returns lse only for
+    autograd and always uses head_dim ** -0.5).
+    """
+    _check_inputs(q, k, v)
+    if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad):
+        raise NotImplementedError("ksa_amd implements the prefill forward only; call it under torch.no_grad()")
+    lib = _lib.lib()
+    b, Sq, Hq, D = q.shape
+    C, S, W = int(chunk_size), int(summary_num), int(sliding_chunk_num)
+    assert C > 0 and S > 0 and W >= 0, "chunk_size/summary_num must be positive, sliding_chunk_num >= 0"
+    q, k, v = _lastdim_contig(q), _lastdim_contig(k), _lastdim_contig(v)
+    kprefix = vprefix = None
+    if summary_pos is not None:
+        assert k.shape[1] == Sq, "with summary_pos, k/v must have the same length as q"
+        P, periodic, rows = _analyse_summary_pos(summary_pos, Sq, C, S)
+        if P > 0 and not periodic:
+            # arbitrary summary positions: gather just the P prefix rows (not the whole K/V)
+            kprefix = torch.empty((b, P, k.shape[2], D), dtype=k.dtype, device=k.device)
+            vprefix = torch.empty_like(kprefix)
+            with torch.cuda.device(q.device):
+                for src, dst in ((k, kprefix), (v, vprefix)):
+                    rc = lib.ksa_copy_rows(src.data_ptr(), dst.data_ptr(), rows.data_ptr(), None, 0, 0,
+                                           P, b, k.shape[2], D, _lib.strides3(src, (0, 2, 1)),
+                                           _lib.strides3(dst, (0, 2, 1)), _lib.stream_ptr(q.device))
+                    _lib.check(rc, "ksa_copy_rows")
+    else:
+        P = k.shape[1] - Sq
+        assert P >= 0, "k/v must be at least as long as q"
+        if P > 0:
+            kprefix, vprefix = k[:, :P], v[:, :P]
+            k, v = k[:, P:], v[:, P:]
+    idx = _cached_index(Sq, C, S, W, P, skip_old_summary, q.device)
+    scale = float(D) ** -0.5 if softmax_scale is None else float(softmax_scale)
+    out, lse = torch.ops.ksa_amd.summary_attn_fwd(
+        q, k, v, kprefix, vprefix, idx[0], idx[1], idx[2], idx[3], C, S, W, P,
+        bool(skip_old_summary), scale, bool(return_lse))
+    return out, (lse if return_lse else None)

@@ -1,0 +1,113 @@
+"""GPU parity of decode attention and the cache row mover against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import to_np
+from oracle import c_oracle
+
+pytestmark = pytest.mark.gpu
+
+ATOL = 2e-2   # bf16 GPU vs fp32 oracle, stated bar
+RTOL_INF = 2e-2
+
+
+def _mk(Bz, Hq, Hkv, Q, D, rows, seed, dtype=torch.bfloat16):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(Bz, Hq, Q, D, generator=g).to(dtype)
+    k = torch.randn(Bz, Hkv, rows, D, generator=g).to(dtype)
+    v = torch.randn(Bz, Hkv, rows, D, generator=g).to(dtype)
+    return q, k, v
+
+
+def _check(q, k, v, start, end, nsplit, scale=None):
+    import ksa_amd
+    dev = torch.device("cuda")
+    Bz = q.shape[0]
+    st = torch.as_tensor(start, dtype=torch.int32, device=dev) if np.ndim(start) else int(start)
+    en = torch.as_tensor(end, dtype=torch.int32, device=dev) if np.ndim(end) else int(end)
+    out = ksa_amd.ksa_decode(q.to(dev), k.to(dev), v.to(dev), st, en, scale=scale, nsplit=nsplit)
+    torch.cuda.synchronize()
+    want = c_oracle.decode(to_np(q), to_np(k), to_np(v), np.broadcast_to(start, (Bz,)),
+                           np.broadcast_to(end, (Bz,)), scale=scale)
+    got = to_np(out)
+    err = np.abs(got - want).max()
+    assert np.isfinite(got).all()
+    assert err <= ATOL and err <= RTOL_INF * np.abs(want).max(), (err, np.abs(want).max())
+
+
+@pytest.mark.parametrize("nsplit", [1, 2, 5, None])
+def test_decode_small(nsplit):
+    q, k, v = _mk(3, 8, 2, 1, 128, 700, seed=0)
+    _check(q, k, v, 0, 700, nsplit)
+
+
+@pytest.mark.parametrize("nsplit", [1, 3])
+def test_decode_per_sequence_ranges(nsplit):
+    """ragged [start, end) per sequence, including one-row and sub-tile slices"""
+    q, k, v = _mk(6, 8, 4, 1, 128, 1000, seed=1)
+    start = np.array([0, 5, 136, 999, 100, 17], np.int32)
+    end = np.array([1000, 6, 900, 1000, 131, 530], np.int32)
+    _check(q, k, v, start, end, nsplit)
+
+
+def test_decode_strided_view_like_hf():
+    """HF hands in cache[:, :, start:end, :] views (non-contiguous batch/head strides)."""
+    import ksa_amd
+    dev = torch.device("cuda")
+    q, k, v = _mk(2, 32, 8, 1, 128, 2000, seed=2)
+    kd, vd = k.to(dev), v.to(dev)
+    kview, vview = kd[:, :, 37:1500, :], vd[:, :, 37:1500, :]
+
+    class M:
+        num_key_value_groups = 4
+    out, w = ksa_amd.decode_attention_forward(M(), q.to(dev), kview, vview, None, scaling=128 ** -0.5)
+    assert w is None and out.shape == (2, 1, 32, 128)
+    want = c_oracle.decode(to_np(q), to_np(k), to_np(v), 37, 1500)
+    assert np.abs(to_np(out) - want).max() <= ATOL
+
+
+def test_decode_boundary_queries():
+    """chunk-boundary step: S = 8 summary queries x g = 4 heads fill one 32-column tile;
+    Q = 9 needs two column blocks."""
+    for Q in (8, 9):
+        q, k, v = _mk(2, 8, 2, Q, 128, 136, seed=3)
+        _check(q, k, v, 0, 136, 1)
+        _check(q, k, v, 0, 136, 2)
+
+
+def test_decode_head_dim_64_and_fp16():
+    q, k, v = _mk(2, 4, 2, 1, 64, 555, seed=4)
+    _check(q, k, v, 3, 555, 2)
+    q, k, v = _mk(2, 4, 2, 1, 128, 555, seed=5, dtype=torch.float16)
+    _check(q, k, v, 3, 555, 1)
+
+
+def test_decode_peaked_softmax():
+    """large scale -> near one-hot attention: exercises the running-max rescale"""
+    q, k, v = _mk(2, 8, 2, 1, 128, 3000, seed=6)
+    _check(q, k, v, 0, 3000, 1, scale=1.0)
+    _check(q, k, v, 0, 3000, 4, scale=1.0)
+
+
+def test_decode_cfg3_shape_subset():
+    """cfg 3 geometry (cap 17288, S=8, C=128, ring 512, 8192 summaries) on 4 of the 64
+    sequences: slice [136 - cbl, 8808)."""
+    Bz, cap = 4, 17288
+    q, k, v = _mk(Bz, 32, 8, 1, 128, cap, seed=7)
+    cbl = np.array([1, 128, 57, 100], np.int32)
+    _check(q, k, v, 136 - cbl, np.full(Bz, 8808, np.int32), None)
+
+
+def test_copy_rows():
+    import ksa_amd
+    from ksa_amd.cache import _move_rows
+    dev = torch.device("cuda")
+    g = torch.Generator().manual_seed(0)
+    src = torch.randn(2, 3, 50, 128, generator=g).bfloat16().to(dev)
+    dst = torch.zeros(2, 3, 80, 128, dtype=torch.bfloat16, device=dev)
+    _move_rows(src, dst, 20, 5, 33)
+    assert torch.equal(dst[:, :, 33:53], src[:, :, 5:25]) and float(dst[:, :, :33].abs().sum()) == 0
+    idx = torch.tensor([7, 3, 49, 0], dtype=torch.int32, device=dev)
+    _move_rows(src, dst, 4, dst_start=60, src_index=idx)
+    assert torch.equal(dst[:, :, 60:64], src[:, :, idx.long()])

@@ -1,0 +1,245 @@
+"""GPU parity of the block index and the prefill forward against the CPU oracle.
+Everything here calls the HIP kernels through the C ABI (ksa_amd -> libksa_hip.so)."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import make_qkv, to_np
+from oracle import c_oracle
+from oracle import ksa_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+# bf16 GPU vs fp32/fp64 CPU oracle: max-abs <= 2e-2 (the stated bar), and, because the
+# benchmark inputs give near-uniform soft-max (outputs ~1e-2), also relative to the
+# largest oracle magnitude.
+ATOL = 2e-2
+RTOL_INF = 2e-2
+
+
+def _index_case(Sq, C, S, W, P, skip_old, tm=128, tn=64):
+    import ksa_amd
+    idx = ksa_amd.compute_block_sparsity(Sq, Sq + P, C, S, W, skip_old, tile_m=tm, tile_n=tn)
+    ref = c_oracle.block_index(Sq, Sq + P, C, S, W, P, skip_old, tm, tn)[:4]
+    M, N = ref[1].shape
+    assert idx[0].shape == (1, 1, M) and idx[1].shape == (1, 1, M, N)
+    assert all(t.dtype == torch.int32 for t in idx)
+    for got, want, name in zip(idx, ref, ("mask_cnt", "mask_idx", "full_cnt", "full_idx")):
+        got = got.cpu().numpy().reshape(want.shape)
+        assert np.array_equal(got, want), f"{name} differs for {(Sq, C, S, W, P, skip_old, tm, tn)}"
+
+
+@pytest.mark.parametrize("W", [0, 1, 3, 4, 1000])
+@pytest.mark.parametrize("skip_old", [False, True])
+def test_index_cfg0(W, skip_old):
+    _index_case(4352, 128, 8, W, 256, skip_old)
+
+
+@pytest.mark.parametrize("case", [
+    # (Sq, C, S, W, P, tm, tn): ragged lengths, partial trailing chunk, tiny chunks, in-line mode
+    (4352 + 77, 128, 8, 3, 256, 128, 64),
+    (1000, 128, 8, 2, 56, 128, 64),
+    (999, 16, 2, 3, 110, 128, 64),
+    (513, 8, 1, 2, 57, 128, 64),
+    (300, 2, 1, 4, 100, 128, 64),
+    (4352, 128, 8, 3, 0, 128, 64),
+    (1234, 32, 4, 1, 0, 128, 64),
+    (2048, 128, 8, 3, 0, 64, 128),
+    (4352, 128, 8, 4, 256, 128, 128),
+])
+@pytest.mark.parametrize("skip_old", [False, True])
+def test_index_odd_shapes(case, skip_old):
+    Sq, C, S, W, P, tm, tn = case
+    _index_case(Sq, C, S, W, P, skip_old, tm, tn)
+
+
+def test_index_cfg1_known_answer():
+    """cfg 1 (256 chunks): totals derived independently of both oracle and kernel."""
+    import ksa_amd
+    for W, (npart, nfull) in {3: (6558, 430), 4: (7076, 445)}.items():
+        idx = ksa_amd.compute_block_sparsity(34816, 36864, 128, 8, W)
+        assert int(idx[0].sum()) == npart and int(idx[2].sum()) == nfull
+    _index_case(34816, 128, 8, 4, 2048, False)
+
+
+def test_index_cfg2_known_answer():
+    """cfg 2 (1024 chunks, 128k): tile totals and the max tiles of one row tile."""
+    import ksa_amd
+    for W, (npart, nfull) in {3: (75438, 4798), 4: (77540, 4861)}.items():
+        idx = ksa_amd.compute_block_sparsity(139264, 147456, 128, 8, W)
+        assert int(idx[0].sum()) == npart and int(idx[2].sum()) == nfull
+        # ascending lists, zero tails
+        mi = idx[1][0, 0]
+        cnt = idx[0][0, 0]
+        ar = torch.arange(mi.shape[1], device=mi.device)[None, :]
+        assert bool((mi[:, 1:] > mi[:, :-1])[ar[:, 1:] < cnt[:, None]].all())
+        assert int(mi[ar >= cnt[:, None]].abs().sum()) == 0
+    assert int((idx[0] + idx[2]).max()) == 139
+
+
+def _run_prefill(q, k, v, C, S, W, summary_pos, skip_old=False, **kw):
+    import ksa_amd
+    dev = torch.device("cuda")
+    sp = None if summary_pos is None else torch.as_tensor(summary_pos, device=dev)
+    out, lse = ksa_amd.summary_attn_func(q[None].to(dev), k[None].to(dev), v[None].to(dev),
+                                         C, S, W, summary_pos=sp, skip_old_summary=skip_old,
+                                         return_lse=True, **kw)
+    torch.cuda.synchronize()
+    return to_np(out[0]), to_np(lse[0])
+
+
+def _compare(got, want, what):
+    err = np.abs(got - want).max()
+    ref = np.abs(want).max()
+    assert np.isfinite(got).all(), f"{what}: non-finite output"
+    assert err <= ATOL, f"{what}: max-abs {err} > {ATOL}"
+    assert err <= RTOL_INF * max(ref, 1e-6), f"{what}: max-abs {err} vs ref magnitude {ref}"
+
+
+@pytest.mark.parametrize("W", [3, 4])
+def test_prefill_cfg0_full_compare(W):
+    """cfg 0: 32 chunks x (128+8), 16 q heads / 8 kv heads, D=128, every output row."""
+    Sq, Hq, Hkv, D, C, S = 4352, 16, 8, 128, 128, 8
+    q, k, v = make_qkv(Sq, Hq, Hkv, D, seed=0)
+    sp = O.summary_positions(Sq, C, S)
+    got, lse = _run_prefill(q, k, v, C, S, W, sp)
+    want, wlse = c_oracle.attention_rows(to_np(q), to_np(k), to_np(v), C, S, W, summary_pos=sp)
+    _compare(got, want, f"cfg0 W={W}")
+    assert np.abs(lse - wlse).max() <= 2e-3
+
+
+@pytest.mark.parametrize("scaled", [False])
+def test_prefill_unscaled_logits(scaled):
+    """N(0,1) q/k (logit sigma ~ 1 after scaling): a peaked soft-max, where a wrong mask
+    or a wrong running max shows up far above the tolerance."""
+    Sq, Hq, Hkv, D, C, S, W = 2176, 8, 2, 128, 128, 8, 3
+    q, k, v = make_qkv(Sq, Hq, Hkv, D, seed=1, scaled=False)
+    q = (q.float() * 3).to(torch.bfloat16)
+    sp = O.summary_positions(Sq, C, S)
+    got, lse = _run_prefill(q, k, v, C, S, W, sp)
+    want, wlse = c_oracle.attention_rows(to_np(q), to_np(k), to_np(v), C, S, W, summary_pos=sp)
+    err = np.abs(got - want).max()
+    assert err <= ATOL * max(1.0, np.abs(want).max()), err
+    assert np.abs(lse - wlse).max() <= 5e-2
+
+
+@pytest.mark.parametrize("case", [
+    # (Sq, Hq, Hkv, D, C, S, W, mode, skip_old)
+    (1088 + 50, 4, 2, 128, 128, 8, 2, "prefix", False),   # trailing partial chunk
+    (1000, 4, 4, 128, 16, 2, 3, "prefix", False),          # small chunks, g = 1
+    (777, 8, 2, 64, 8, 1, 2, "prefix", False),             # head_dim 64, ragged
+    (1360, 4, 1, 128, 128, 8, 1, "inline", False),         # in-line summaries (P = 0)
+    (1360, 4, 2, 128, 128, 8, 2, "prefix", True),          # skip_old_summary
+    (1360, 4, 2, 128, 128, 8, 2, "inline", True),
+    (1360, 4, 2, 128, 128, 8, 2, "physical", False),       # k/v already carry the prefix
+    (130, 2, 2, 128, 128, 8, 0, "prefix", False),          # shorter than one block + tail
+    (64, 2, 1, 128, 128, 8, 4, "prefix", False),           # no summaries at all
+])
+def test_prefill_variants(case):
+    Sq, Hq, Hkv, D, C, S, W, mode, skip_old = case
+    q, k, v = make_qkv(Sq, Hq, Hkv, D, seed=2, scaled=False)
+    sp = O.summary_positions(Sq, C, S)
+    qn, kn, vn = to_np(q), to_np(k), to_np(v)
+    if mode == "prefix":
+        got, lse = _run_prefill(q, k, v, C, S, W, sp, skip_old)
+        want, wlse = c_oracle.attention_rows(qn, kn, vn, C, S, W, summary_pos=sp, skip_old=skip_old)
+    elif mode == "inline":
+        got, lse = _run_prefill(q, k, v, C, S, W, None, skip_old)
+        want, wlse = c_oracle.attention_rows(qn, kn, vn, C, S, W, summary_pos=None, skip_old=skip_old)
+    else:
+        spt = torch.as_tensor(sp)
+        kk = torch.cat([k[spt], k]); vv = torch.cat([v[spt], v])
+        got, lse = _run_prefill(q, kk, vv, C, S, W, None, skip_old)
+        want, wlse = c_oracle.attention_rows(qn, kn, vn, C, S, W, summary_pos=sp, skip_old=skip_old)
+    err = np.abs(got - want).max()
+    assert err <= ATOL * max(1.0, np.abs(want).max()), (case, err)
+    assert np.abs(lse - wlse).max() <= 5e-2
+
+
+def test_prefill_nonperiodic_summary_pos():
+    """summary_pos that is not the periodic pattern takes the gathered-prefix route; the
+    mask rule still assumes the periodic layout, exactly as the reference's does."""
+    Sq, Hq, Hkv, D, C, S, W = 1360, 4, 2, 128, 128, 8, 2
+    q, k, v = make_qkv(Sq, Hq, Hkv, D, seed=3, scaled=False)
+    rng = np.random.default_rng(0)
+    sp = np.zeros(Sq, bool)
+    sp[rng.choice(Sq, 80, replace=False)] = True
+    got, _ = _run_prefill(q, k, v, C, S, W, sp)
+    want, _ = c_oracle.attention_rows(to_np(q), to_np(k), to_np(v), C, S, W, summary_pos=sp)
+    assert np.abs(got - want).max() <= ATOL * max(1.0, np.abs(want).max())
+
+
+def test_prefill_visibility_probe():
+    """Q = K = 0 makes every visible key equally weighted; V = one-hot of the key's
+    position class.  Output row i is then exactly (count of class)/n_i on its visible set,
+    so a single mis-masked element changes a value by 1/n_i >> tolerance."""
+    Sq, Hq, Hkv, D, C, S, W = 2720, 2, 1, 128, 128, 8, 3
+    q = torch.zeros(Sq, Hq, D, dtype=torch.bfloat16)
+    k = torch.zeros(Sq, Hkv, D, dtype=torch.bfloat16)
+    v = torch.zeros(Sq, Hkv, D, dtype=torch.bfloat16)
+    v[torch.arange(Sq), 0, torch.arange(Sq) % D] = 1.0
+    sp = O.summary_positions(Sq, C, S)
+    got, _ = _run_prefill(q, k, v, C, S, W, sp)
+    P = int(sp.sum())
+    vis = O.dense_mask_predicate(Sq, C, S, W, P)
+    vfull = np.concatenate([to_np(v)[sp], to_np(v)], axis=0)[:, 0, :]
+    want = (vis.astype(np.float64) @ vfull) / vis.sum(axis=1, keepdims=True)
+    # values are k/n with n up to ~700: bf16 rounding of P (8 bits) bounds the error
+    assert np.abs(got[:, 0] - want).max() <= 4e-3
+    assert np.abs(got[:, 1] - want).max() <= 4e-3
+
+
+def test_prefill_cfg1_sampled_rows():
+    """cfg 1 (32k text tokens, 32/8 heads): rows of the first and last two chunks, offsets
+    {0, C-1, C, B-1} of 64 random chunks and 1024 random rows against the oracle."""
+    Sq, Hq, Hkv, D, C, S, W = 34816, 32, 8, 128, 128, 8, 4
+    q, k, v = make_qkv(Sq, Hq, Hkv, D, seed=0)
+    sp = O.summary_positions(Sq, C, S)
+    got, lse = _run_prefill(q, k, v, C, S, W, sp)
+    rng = np.random.default_rng(0)
+    B = C + S
+    rows = set(range(0, 2 * B)) | set(range(Sq - 2 * B, Sq))
+    for c in rng.choice(Sq // B, 64, replace=False):
+        rows |= {c * B, c * B + C - 1, c * B + C, c * B + B - 1}
+    rows |= set(rng.choice(Sq, 1024, replace=False).tolist())
+    rows = np.array(sorted(rows), np.int32)
+    want, wlse = c_oracle.attention_rows(to_np(q), to_np(k), to_np(v), C, S, W, summary_pos=sp, rows=rows)
+    _compare(got[rows], want, "cfg1 sampled rows")
+    assert np.abs(lse[:, rows] - wlse).max() <= 2e-3
+
+
+def test_prefill_batch_and_fp16():
+    Sq, Hq, Hkv, D, C, S, W = 680, 4, 2, 128, 128, 8, 1
+    import ksa_amd
+    dev = torch.device("cuda")
+    outs = []
+    qs, ks, vs = [], [], []
+    for b in range(2):
+        q, k, v = make_qkv(Sq, Hq, Hkv, D, seed=10 + b, scaled=False)
+        qs.append(q.half()); ks.append(k.half()); vs.append(v.half())
+    sp = O.summary_positions(Sq, C, S)
+    out, _ = ksa_amd.summary_attn_func(torch.stack(qs).to(dev), torch.stack(ks).to(dev),
+                                       torch.stack(vs).to(dev), C, S, W,
+                                       summary_pos=torch.as_tensor(sp, device=dev))
+    assert out.dtype == torch.float16
+    for b in range(2):
+        want, _ = c_oracle.attention_rows(to_np(qs[b]), to_np(ks[b]), to_np(vs[b]), C, S, W, summary_pos=sp)
+        assert np.abs(to_np(out[b]) - want).max() <= 5e-3 * max(1.0, np.abs(want).max())
+
+
+def test_prefill_rejects_bad_inputs():
+    import ksa_amd
+    dev = torch.device("cuda")
+    q = torch.zeros(1, 136, 4, 128, device=dev, dtype=torch.float32)
+    with pytest.raises(AssertionError):
+        ksa_amd.summary_attn_func(q, q, q, 128, 8, 1)
+    q = q.bfloat16()
+    k = torch.zeros(1, 136, 3, 128, device=dev, dtype=torch.bfloat16)
+    with pytest.raises(AssertionError):
+        ksa_amd.summary_attn_func(q, k, k, 128, 8, 1)
+    q96 = torch.zeros(1, 136, 4, 96, device=dev, dtype=torch.bfloat16)
+    with pytest.raises(ksa_amd.KsaError):
+        ksa_amd.summary_attn_func(q96, q96, q96, 128, 8, 1)
+    qg = q.clone().requires_grad_(True)
+    with pytest.raises(NotImplementedError):
+        ksa_amd.summary_attn_func(qg, q, q, 128, 8, 1)
