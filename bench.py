@@ -1,0 +1,256 @@
+#!/usr/bin/env python3
+"""Benchmark of the two KSA attention hot paths on one MI355X.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--prefill-chunks 1024]
+
+Prints ONE JSON line.  A "step" is one prefill forward of a single Summary-Attention
+layer on the 128k configuration (1024 chunks x (128 text + 8 summary) rows, 32 query /
+8 KV heads, head_dim 128, bf16); `value` is its non-empty-block TFLOP/s.  The decode
+attention step over the ring-buffer cache (batch 64, 128k logical context) is timed in a
+second region of the same K/W and reported under "decode".  Inputs are synthetic, seeded,
+and resident in HBM before any timed region.  The block index is built once before the
+timed region (the reference caches it the same way); reading the summary prefix is inside.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E
+
+
+def prefill_inputs(chunks, Hq, Hkv, D, C, S, device, seed):
+    import torch
+    Sq = chunks * (C + S)
+    g = torch.Generator(device=device).manual_seed(seed)
+    scale = D ** -0.5
+
+    def draw(h):
+        t = torch.empty(1, Sq, h, D, dtype=torch.bfloat16, device=device)
+        step = 8192
+        for r in range(0, Sq, step):
+            n = min(step, Sq - r)
+            t[0, r:r + n] = (torch.randn(n, h, D, generator=g, device=device) * scale).to(torch.bfloat16)
+        return t
+
+    q, k, v = draw(Hq), draw(Hkv), draw(Hkv)
+    i = torch.arange(Sq, device=device)
+    summary_pos = (i % (C + S)) >= C
+    return q, k, v, summary_pos
+
+
+def time_region(fn, steps, warmup):
+    """Runs `warmup` untimed and exactly `steps` timed calls; returns (wall seconds,
+    device milliseconds from HIP events recorded on the launch stream)."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    return t1 - t0, e0.elapsed_time(e1)
+
+
+def cpu_baseline_prefill(chunks, Hq, Hkv, D, C, S, W, tiles_per_mtile, budget_s=12.0):
+    """The reference's CPU path (block mode, restated in oracle/cpu_path.py) on a bounded
+    sample of 4096-row query blocks; rate in the same non-empty-block TFLOP/s unit."""
+    import torch
+    from oracle import cpu_path
+    Sq = chunks * (C + S)
+    torch.manual_seed(0)
+    scale = D ** -0.5
+    k = (torch.randn(Sq, Hkv, D) * scale).bfloat16().float()
+    v = (torch.randn(Sq, Hkv, D) * scale).bfloat16().float()
+    nblk = -(-Sq // cpu_path.BLOCK_ROWS)
+    pick = sorted({0, nblk // 2, nblk - 1})
+    # non-empty 128 x 64 tiles of the sampled rows come from the (parity-checked) block index
+    done_tiles, t_used, blocks = 0, 0.0, []
+    for bi in pick:
+        q0 = bi * cpu_path.BLOCK_ROWS
+        q1 = min(Sq, q0 + cpu_path.BLOCK_ROWS)
+        q = (torch.randn(q1 - q0, Hq, D) * scale).bfloat16().float()
+        t0 = time.perf_counter()
+        cpu_path.block_mode_rows(q, k, v, q0, C, S, W)
+        dt = time.perf_counter() - t0
+        tiles = int(tiles_per_mtile[q0 // 128:-(-q1 // 128)].sum())
+        done_tiles += tiles
+        t_used += dt
+        blocks.append(bi)
+        if t_used > budget_s:
+            break
+    flops = 4.0 * 128 * 64 * D * Hq * done_tiles
+    return {
+        "value": flops / t_used / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"query blocks {blocks} of {nblk} (4096 rows each) of the same workload, "
+                  f"fp32 torch SDPA block mode with KV expanded to {Hq} heads, {t_used:.1f} s",
+    }
+
+
+def cpu_baseline_decode(Hq, Hkv, D, rows, nseq=2):
+    import torch
+    from oracle import cpu_path
+    torch.manual_seed(0)
+    q = torch.randn(nseq, Hq, 1, D)
+    k = torch.randn(nseq, Hkv, rows, D)
+    v = torch.randn(nseq, Hkv, rows, D)
+    cpu_path.decode_sdpa(q, k, v, Hq // Hkv)
+    t0 = time.perf_counter()
+    reps = 3
+    for _ in range(reps):
+        cpu_path.decode_sdpa(q, k, v, Hq // Hkv)
+    dt = (time.perf_counter() - t0) / reps
+    return {"us_per_sequence": dt / nseq * 1e6, "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"{nseq} of 64 sequences, {rows} rows, repeat_kv + fp32 torch SDPA"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--prefill-chunks", type=int, default=1024, help="1024 = 128k text tokens (cfg 2)")
+    ap.add_argument("--sliding-chunk-num", type=int, default=4)
+    ap.add_argument("--decode-batch", type=int, default=64)
+    ap.add_argument("--decode-splits", type=int, default=0, help="0 = library heuristic")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--skip-decode", action="store_true")
+    ap.add_argument("--skip-prefill", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (see DESIGN.md, "
+              "'How the paths would shard'); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import ksa_amd
+    from ksa_amd import _lib
+
+    assert torch.cuda.is_available(), "bench.py needs an MI355X"
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    C, S, D, Hq, Hkv = 128, 8, 128, 32, 8
+    W = args.sliding_chunk_num
+    result = {
+        "metric": "prefill non-empty-block TFLOP/s @128k; decode step us + HBM GB/s (bs=64)",
+        "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic (seed 0; q,k,v ~ N(0,1)/sqrt(128) for prefill, N(0,1) for decode)",
+        "device": torch.cuda.get_device_name(0), "cu_count": _lib.lib().ksa_device_cu_count(),
+    }
+
+    # ------------------------------------------------------------------ prefill
+    if not args.skip_prefill:
+        chunks = args.prefill_chunks
+        Sq = chunks * (C + S)
+        P = chunks * S
+        q, k, v, sp = prefill_inputs(chunks, Hq, Hkv, D, C, S, dev, seed=0)
+        idx = ksa_amd.compute_block_sparsity(Sq, Sq + P, C, S, W)
+        tiles_per_mtile = (idx[0] + idx[2]).flatten().cpu().numpy()
+        tiles = int(tiles_per_mtile.sum())
+        flops = 4.0 * 128 * 64 * D * Hq * tiles
+        t_idx0 = time.perf_counter()
+        ksa_amd.compute_block_sparsity(Sq, Sq + P, C, S, W)
+        torch.cuda.synchronize()
+        idx_ms = (time.perf_counter() - t_idx0) * 1e3
+
+        def step():
+            ksa_amd.summary_attn_func(q, k, v, C, S, W, summary_pos=sp)
+
+        wall, dev_ms = time_region(step, args.steps, args.warmup)
+        ms = wall * 1e3 / args.steps
+        kern_ms = dev_ms / args.steps
+        result.update({
+            "value": flops / (wall / args.steps) / 1e12,
+            "ms_per_step": ms,
+            "config": {"workload": f"cfg2-prefill-128k" if chunks == 1024 else f"prefill-{chunks}-chunks",
+                       "chunks": chunks, "seqlen_q": Sq, "prefix_summaries": P, "q_heads": Hq,
+                       "kv_heads": Hkv, "head_dim": D, "chunk_size": C, "summary_num": S,
+                       "sliding_chunk_num": W, "non_empty_tiles_128x64": tiles,
+                       "non_empty_block_tflop": flops / 1e12, "block_index_ms": idx_ms},
+            "roofline": {"bound": "mfma", "achieved": flops / (kern_ms * 1e-3) / 1e12,
+                         "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                         "frac": flops / (kern_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+                         "traffic": None, "kernel": "ksa_prefill_kernel<bf16,128>",
+                         "kernel_ms": kern_ms},
+        })
+        del q, k, v, sp
+        torch.cuda.empty_cache()
+
+    # ------------------------------------------------------------------ decode
+    if not args.skip_decode:
+        Bz = args.decode_batch
+        n_chunks_done = 1024
+        ws = W * C
+        n_sum = n_chunks_done * S
+        cap = S + C + ws + n_sum + max(512, n_sum + 256)
+        g = torch.Generator(device=dev).manual_seed(1)
+        kc = torch.empty(Bz, Hkv, cap, D, dtype=torch.bfloat16, device=dev)
+        vc = torch.empty_like(kc)
+        for b in range(Bz):
+            kc[b] = torch.randn(Hkv, cap, D, generator=g, device=dev).to(torch.bfloat16)
+            vc[b] = torch.randn(Hkv, cap, D, generator=g, device=dev).to(torch.bfloat16)
+        qd = torch.randn(Bz, Hq, 1, D, generator=g, device=dev).to(torch.bfloat16)
+        cbl = torch.randint(0, C, (Bz,), generator=g, device=dev, dtype=torch.int32) + 1  # after update_text
+        start = (S + C - cbl).to(torch.int32)
+        end = torch.full((Bz,), S + C + ws + n_sum - min(W * S, n_sum), dtype=torch.int32, device=dev)
+        L = (end - start).to(torch.int64)
+        bytes_step = int((2 * L * Hkv * D * 2 + 2 * Hq * D * 2).sum())
+        nsplit = args.decode_splits or _lib.lib().ksa_decode_auto_splits(Bz, Hkv, cap)
+
+        def dstep():
+            ksa_amd.ksa_decode(qd, kc, vc, start, end, nsplit=nsplit)
+
+        wall, dev_ms = time_region(dstep, args.steps, args.warmup)
+        us = dev_ms * 1e3 / args.steps
+        result["decode"] = {
+            "workload": "cfg3-decode-bs64-128k" if Bz == 64 else f"decode-bs{Bz}",
+            "batch": Bz, "rows_per_sequence_mean": float(L.float().mean()), "cache_rows": cap,
+            "nsplit": nsplit, "us_per_step": us, "us_per_step_wall": wall * 1e6 / args.steps,
+            "algorithmic_bytes": bytes_step, "hbm_gbps": bytes_step / (us * 1e-6) / 1e9,
+            "roofline": {"bound": "hbm", "achieved": bytes_step / (us * 1e-6) / 1e9,
+                         "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+                         "frac": bytes_step / (us * 1e-6) / 1e9 / PEAK_HBM_GBPS, "traffic": None,
+                         "kernel": "ksa_decode_kernel<bf16,128> (+ merge when nsplit > 1)"},
+        }
+        if args.skip_prefill:
+            result.update({"value": result["decode"]["hbm_gbps"], "unit": "GB/s",
+                           "ms_per_step": us / 1e3,
+                           "config": {"workload": result["decode"]["workload"]},
+                           "roofline": result["decode"]["roofline"]})
+        del kc, vc
+        torch.cuda.empty_cache()
+
+    # ------------------------------------------------------------------ CPU baseline
+    if not args.no_cpu_baseline:
+        try:
+            Sq_ = args.prefill_chunks * (C + S)
+            ix = ksa_amd.compute_block_sparsity(Sq_, Sq_ + args.prefill_chunks * S, C, S, W)
+            cb = cpu_baseline_prefill(args.prefill_chunks, Hq, Hkv, D, C, S, W,
+                                      (ix[0] + ix[2]).flatten().cpu().numpy())
+            if not args.skip_decode:
+                cb["decode"] = cpu_baseline_decode(Hq, Hkv, D, 8672 + 64)
+            result["cpu_baseline"] = cb
+        except Exception as e:  # the baseline is a reported extra, never the measured path
+            result["cpu_baseline"] = {"error": repr(e)}
+
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
