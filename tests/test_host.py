@@ -1,0 +1,184 @@
+"""CPU-side checks of the product's host logic: the C ABI loads and exports everything
+include/ksa_hip.h declares, rejects bad arguments before any launch, the closed-form
+visibility rule used by the kernels equals the oracle predicate, and the cache class keeps
+the reference's bookkeeping (checked against the oracle's integer model with a host row
+mover injected by the test — the product itself has none)."""
+import ctypes
+import os
+import re
+import types
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import ksa_oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    from ksa_amd import _lib
+    L = _lib.lib()
+    header = open(os.path.join(ROOT, "include", "ksa_hip.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(ksa_[a-z0-9_]+)\s*\(", header))
+    assert declared, "no declarations found"
+    assert declared == set(_lib.EXPORTS), declared ^ set(_lib.EXPORTS)
+    for name in declared:
+        assert getattr(L, name) is not None
+    assert L.ksa_version() >= 100
+    assert b"ok" == L.ksa_error_string(0)
+
+
+def test_error_codes_before_launch():
+    from ksa_amd import _lib
+    L = _lib.lib()
+    # bad sizes / null pointers are rejected without touching a device
+    assert L.ksa_block_index(0, 10, 128, 8, 3, 10, 0, 128, 64, None, None, None, None, None) == -1
+    assert L.ksa_block_index(100, 110, 128, 8, 3, 9, 0, 128, 64, None, None, None, None, None) == -1
+    assert L.ksa_block_index(100, 110, 128, 8, 3, 10, 0, 128, 64, None, None, None, None, None) == -2
+    null3 = ctypes.cast(None, ctypes.POINTER(ctypes.c_int64))
+    assert L.ksa_prefill_fwd(None, None, None, None, None, None, None, 1, 128, 4, 2, 128, 0, null3, null3,
+                             null3, null3, null3, null3, 128, 8, 3, 0, 0, None, None, None, None, 2,
+                             1.0, None) == -2
+    assert L.ksa_decode_fwd(None, None, None, None, None, None, 0, 10, 1, 4, 2, 1, 128, 0, null3, null3,
+                            null3, null3, 1.0, 1, None, 0, None) == -2
+    assert L.ksa_decode_workspace_bytes(64, 32, 8, 1, 128, 1) == 0
+    assert L.ksa_decode_workspace_bytes(64, 32, 8, 1, 128, 2) == 64 * 8 * 2 * 32 * 130 * 4
+    assert L.ksa_decode_auto_splits(64, 8, 17288) == 2
+    assert L.ksa_decode_auto_splits(1, 8, 100) == 1
+    assert 1 <= L.ksa_decode_auto_splits(1, 8, 100000) <= 64
+
+
+@pytest.mark.parametrize("P_mode", ["prefix", "inline"])
+def test_closed_form_counts_equal_predicate(P_mode):
+    """ksa_count_visible (csrc/ksa_mask.h, the rule both the index kernel and the prefill
+    mask are built on) against brute force over the oracle predicate."""
+    from ksa_amd import _lib
+    L = _lib.lib()
+    rng = np.random.default_rng(1)
+    for _ in range(60):
+        C, S = int(rng.integers(1, 24)), int(rng.integers(1, 6))
+        W = int(rng.integers(0, 6))
+        n = int(rng.integers(1, 9))
+        Sq = n * (C + S) + int(rng.integers(0, C + 1))
+        P = (Sq // (C + S)) * S if P_mode == "prefix" else 0
+        Sk = Sq + P
+        skip = int(rng.integers(0, 2))
+        vis = O.dense_mask_predicate(Sq, C, S, W, P, bool(skip))
+        cum = np.concatenate([np.zeros((Sq, 1), np.int64), np.cumsum(vis, axis=1)], axis=1)
+        for _ in range(40):
+            q = int(rng.integers(0, Sq))
+            a = int(rng.integers(0, Sk))
+            b = int(rng.integers(a, Sk + 1))
+            got = L.ksa_debug_count_visible(q, a, b, C, S, W, P, skip, Sq, Sk)
+            assert got == cum[q, b] - cum[q, a], (C, S, W, P, skip, q, a, b)
+
+
+def _host_mover(src, dst, nrows, src_start=0, dst_start=0, src_index=None):
+    if nrows <= 0:
+        return
+    rows = src_index.long() if src_index is not None else torch.arange(src_start, src_start + nrows)
+    dst[:, :, dst_start:dst_start + nrows, :] = src[:, :, rows[:nrows], :].clone()
+
+
+def _make_cache(C, S, scns):
+    from ksa_amd.cache import Qwen3RingBufferCache
+    cfg = types.SimpleNamespace(summary_chunk_size=C, summary_token_num=S, num_hidden_layers=len(scns))
+
+    class HostCache(Qwen3RingBufferCache):
+        _move_rows = staticmethod(_host_mover)
+    return HostCache(cfg, scns)
+
+
+@pytest.mark.parametrize("C,S", [(4, 2), (8, 1)])
+@pytest.mark.parametrize("n_prefill", [1, 7, 16, 37])
+def test_cache_bookkeeping_matches_model(C, S, n_prefill):
+    """Drives the product cache class and the oracle's integer model with the same tagged
+    rows through prefill, reorganisation, decode steps and chunk boundaries."""
+    scns = [2, 3, 1000]                # last layer is a large-window layer
+    cache = _make_cache(C, S, scns)
+    assert cache.is_large_window == [False, True, True]
+    B = C + S
+    n_full = n_prefill // C
+    Sq = n_full * B + n_prefill % C
+    sp = O.summary_positions(Sq, C, S)
+    D, H = 8, 2
+    tags = torch.arange(Sq, dtype=torch.float32)
+    kv = tags[None, None, :, None].expand(1, H, Sq, D).to(torch.bfloat16).contiguous()
+    models = [O.RingBufferModel(C, S, scn, large) for scn, large in zip(scns, cache.is_large_window)]
+    spt = torch.from_numpy(sp)[None]
+    for layer in range(3):
+        k_all, v_all = cache.update(kv, kv, layer, {"summary_mask": spt})
+        assert k_all.shape[2] == Sq
+    # as in the reference, a small-window layer reports 0 until the cache is reorganised
+    assert cache.get_true_token_num() == n_prefill and cache.get_seq_length(0) == 0 and cache.get_seq_length(1) == Sq
+    cache.reorganize_after_prefill(spt)
+    for m in models:
+        m.reorganize_after_prefill(np.arange(Sq), sp)
+    pos = Sq
+    n_text = n_prefill
+
+    def check():
+        for layer, m in enumerate(models):
+            a, b = m.attention_range()
+            assert cache.attention_range(layer) == (a, b)
+            k, v = cache.get_attention_kv(layer)
+            assert k.shape[2] == b - a
+            assert sorted(k[0, 0, :, 0].float().tolist()) == sorted(m.buf[a:b].tolist())
+            assert cache._capacity[layer] == m.cap == cache.key_cache[layer].shape[2]
+        assert cache.get_true_token_num() == n_text
+
+    check()
+    for _ in range(3 * C + 1):
+        row = torch.full((1, H, 1, D), float(pos), dtype=torch.bfloat16)
+        for layer, m in enumerate(models):
+            cache.update_text(row, row, layer)
+            m.update_text(pos)
+        n_text += 1
+        pos += 1
+        check()
+        if n_text % C == 0:
+            stags = np.arange(pos, pos + S)
+            srow = torch.from_numpy(stags.astype(np.float32))[None, None, :, None].expand(1, H, S, D).to(torch.bfloat16)
+            for layer, m in enumerate(models):
+                ks, vs = cache.get_summary_attention_kv(layer, srow, srow)
+                assert sorted(ks[0, 0, :, 0].float().tolist()) == list(range(pos - C, pos + S))
+                cache.update_summary(srow, srow, layer)
+                m.update_summary(stags)
+            pos += S
+            assert cache.get_cur_chunk_size() == B
+            cache.reset_chunk_counter()
+            assert cache.get_cur_chunk_size() == 0
+            check()
+
+
+def test_cache_summary_growth():
+    """Summary region overflows its headroom -> buffer grows to the right, rows keep their place."""
+    C, S = 2, 1
+    cache = _make_cache(C, S, [1])
+    cache._SUMMARY_INIT_CAP = 4
+    model = O.RingBufferModel(C, S, 1)
+    model.SUMMARY_INIT_CAP = 4
+    Sq = 3
+    sp = O.summary_positions(Sq, C, S)
+    kv = torch.arange(Sq, dtype=torch.float32)[None, None, :, None].expand(1, 1, Sq, 8).to(torch.bfloat16).contiguous()
+    cache.update(kv, kv, 0, {"summary_mask": torch.from_numpy(sp)[None]})
+    cache.reorganize_after_prefill(torch.from_numpy(sp)[None])
+    model.reorganize_after_prefill(np.arange(Sq), sp)
+    pos = Sq
+    for step in range(1200):
+        row = torch.full((1, 1, 1, 8), float(pos % 251), dtype=torch.bfloat16)
+        cache.update_text(row, row, 0)
+        model.update_text(pos % 251)
+        pos += 1
+        if cache._chunk_buf_len[0] == C:
+            srow = torch.full((1, 1, S, 8), float(pos % 251), dtype=torch.bfloat16)
+            cache.update_summary(srow, srow, 0)
+            model.update_summary([pos % 251])
+            pos += 1
+    assert cache._capacity[0] == model.cap > 300
+    a, b = model.attention_range()
+    assert cache.attention_range(0) == (a, b)
+    assert cache.key_cache[0][0, 0, a:b, 0].float().tolist() == [float(x) for x in model.buf[a:b]]
