@@ -53,12 +53,10 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_decode_kernel(const DecodePar
     constexpr int KS = D / 16;
     constexpr int DB = D / 32;
     constexpr int KROW = D + 8;
-    constexpr int VROW = kRows + 8;
+    constexpr int VROW = D + 16;
     constexpr int CPR = D / 8;
-    constexpr int KLD = (kRows * CPR) / 64;          // K loads per lane
-    constexpr int VUNITS = (kRows / 4) * CPR;
-    constexpr int VLD = (VUNITS + 63) / 64;
-    constexpr int kStage = kRows * KROW + D * VROW;  // elements of one wave's staging area
+    constexpr int KLD = (kRows * CPR) / 64;          // K (and V) loads per lane
+    constexpr int kStage = kRows * (KROW + VROW);    // elements of one wave's staging area
     constexpr int kMergeFloats = kWaves * 32 * (D + 2);
     constexpr int kSmemBytes = (kWaves * kStage * 2 > kMergeFloats * 4) ? kWaves * kStage * 2
                                                                         : kMergeFloats * 4;
@@ -109,7 +107,7 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_decode_kernel(const DecodePar
     const int last_row = max(r_end - 1, r_begin);
 
     u32x4 kreg[KLD];
-    u32x4 vreg[VLD][4];
+    u32x4 vreg[KLD];
 
     auto load_tile = [&](int row0) {
 #pragma unroll
@@ -117,18 +115,7 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_decode_kernel(const DecodePar
             const int u = lane + 64 * i;
             const int row = min(row0 + u / CPR, last_row);
             kreg[i] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)row * p.k_rs + 8 * (u % CPR));
-        }
-#pragma unroll
-        for (int i = 0; i < VLD; ++i) {
-            const int u = lane + 64 * i;
-            if (u < VUNITS) {
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int row = min(row0 + 4 * (u / CPR) + r, last_row);
-                    vreg[i][r] =
-                        *reinterpret_cast<const u32x4*>(vbase + (int64_t)row * p.v_rs + 8 * (u % CPR));
-                }
-            }
+            vreg[i] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)row * p.v_rs + 8 * (u % CPR));
         }
     };
 
@@ -150,11 +137,7 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_decode_kernel(const DecodePar
         for (int i = 0; i < KLD; ++i) {
             const int u = lane + 64 * i;
             *reinterpret_cast<u32x4*>(Kw + (u / CPR) * KROW + 8 * (u % CPR)) = kreg[i];
-        }
-#pragma unroll
-        for (int i = 0; i < VLD; ++i) {
-            const int u = lane + 64 * i;
-            if (u < VUNITS) ksa_store_vt<VROW>(Vw, 8 * (u % CPR), ksa_vt_pos(u / CPR), vreg[i]);
+            *reinterpret_cast<u32x4*>(Vw + (u / CPR) * VROW + 8 * (u % CPR)) = vreg[i];
         }
         ksa_wave_lds_fence();
         const int next = row0 + kWaves * kRows;
@@ -203,8 +186,7 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_decode_kernel(const DecodePar
         for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
             for (int b = 0; b < DB; ++b) {
-                const u32x4 a =
-                    *reinterpret_cast<const u32x4*>(Vw + (b * 32 + lq) * VROW + 16 * ks + 8 * lh);
+                const u32x4 a = ksa_read_vt_frag<VROW>(Vw, ks, b, lq, lh);
                 oacc[b] = Ops::mfma(a, pf[ks], oacc[b]);
             }
     }

@@ -11,8 +11,8 @@
 //
 // One workgroup (4 waves) owns a 128-row query tile of one query head; wave w owns
 // rows 32w .. 32w+31.  It walks the tile's non-empty key tiles (64 keys each) taken
-// from the block index, staging K row-major and V transposed in LDS (two buffers),
-// see ksa_tile.h for the operand layouts.  The summary prefix of the key axis is
+// from the block index, staging K and V row-major in LDS (two buffers); V is transposed
+// on the way out of LDS by ds_read_b64_tr_b16, see ksa_tile.h for the operand layouts.  The summary prefix of the key axis is
 // read in place from the in-line summary rows (or from a separate prefix buffer),
 // never concatenated.
 //
@@ -64,14 +64,12 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
     constexpr int KS = D / 16;       // contraction steps of K Q^T
     constexpr int DB = D / 32;       // 32-row blocks of O^T
     constexpr int KROW = D + 8;      // padded LDS row of K (elements)
-    constexpr int VROW = kTileN + 8;  // padded LDS row of V^T
+    constexpr int VROW = D + 16;     // padded LDS row of V (stride = 8 banks mod 64)
     constexpr int CPR = D / 8;       // 16-byte chunks per K/V row
-    constexpr int KLD = (kTileN * CPR) / kThreads;            // K loads per thread
-    constexpr int VUNITS = (kTileN / 4) * CPR;                // (4 keys x 8 dims) units
-    constexpr int VLD = (VUNITS + kThreads - 1) / kThreads;   // V units per thread
+    constexpr int KLD = (kTileN * CPR) / kThreads;  // K (and V) loads per thread
 
     __shared__ __attribute__((aligned(16))) uint16_t Ks[2][kTileN * KROW];
-    __shared__ __attribute__((aligned(16))) uint16_t Vt[2][D * VROW];
+    __shared__ __attribute__((aligned(16))) uint16_t Vs[2][kTileN * VROW];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -113,7 +111,7 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
     const int32_t* flist = p.full_idx + (int64_t)mt * p.idx_stride;
 
     u32x4 kreg[KLD];
-    u32x4 vreg[VLD][4];
+    u32x4 vreg[KLD];
 
     auto row_ptrs = [&](int kv, const uint16_t*& kr, const uint16_t*& vr) {
         kv = min(kv, mk.Sk - 1);
@@ -141,19 +139,7 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
             const uint16_t *kr, *vr;
             row_ptrs(n0 + row, kr, vr);
             kreg[i] = *reinterpret_cast<const u32x4*>(kr + 8 * c);
-        }
-#pragma unroll
-        for (int i = 0; i < VLD; ++i) {
-            const int u = tid + kThreads * i;
-            if (u < VUNITS) {
-                const int kv4 = u / CPR, d8 = u % CPR;
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const uint16_t *kr, *vr;
-                    row_ptrs(n0 + 4 * kv4 + r, kr, vr);
-                    vreg[i][r] = *reinterpret_cast<const u32x4*>(vr + 8 * d8);
-                }
-            }
+            vreg[i] = *reinterpret_cast<const u32x4*>(vr + 8 * c);
         }
     };
 
@@ -163,14 +149,7 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
             const int u = tid + kThreads * i;
             const int row = u / CPR, c = u % CPR;
             *reinterpret_cast<u32x4*>(&Ks[buf][row * KROW + 8 * c]) = kreg[i];
-        }
-#pragma unroll
-        for (int i = 0; i < VLD; ++i) {
-            const int u = tid + kThreads * i;
-            if (u < VUNITS) {
-                const int kv4 = u / CPR, d8 = u % CPR;
-                ksa_store_vt<VROW>(Vt[buf], 8 * d8, ksa_vt_pos(kv4), vreg[i]);
-            }
+            *reinterpret_cast<u32x4*>(&Vs[buf][row * VROW + 8 * c]) = vreg[i];
         }
     };
 
@@ -270,8 +249,7 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
         for (int ks = 0; ks < 4; ++ks) {
 #pragma unroll
             for (int b = 0; b < DB; ++b) {
-                const u32x4 a = *reinterpret_cast<const u32x4*>(
-                    &Vt[buf][(b * 32 + lq) * VROW + 16 * ks + 8 * lh]);
+                const u32x4 a = ksa_read_vt_frag<VROW>(Vs[buf], ks, b, lq, lh);
                 oacc[b] = Ops::mfma(a, pf[ks], oacc[b]);
             }
         }

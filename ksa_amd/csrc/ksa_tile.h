@@ -11,9 +11,11 @@
 //
 // For the second product the contraction index is the key position.  The C layout
 // above hands lane (q, h) the keys {16*ks + 8*a + 4*h + r : a<2, r<4} of k-step ks as
-// its 8 B-operand elements e = 4*a + r, so V^T is stored in LDS with key position
-//   pos(kv) = 16*(kv/16) + 8*h + 4*a + r      for kv = 16*(kv/16) + 8*a + 4*h + r
-// and the A operand of lane (d, h) is the 16 contiguous bytes at V^T[d][16*ks + 8*h].
+// its 8 B-operand elements e = 4*a + r.  V stays row-major in LDS ([key][dim], like K) and
+// the matching A operand of lane (d, h) -- V[those 8 keys][d] -- is fetched with two
+// ds_read_b64_tr_b16: within each group of 16 lanes, lane t supplies the address of 4
+// consecutive dims of key (K0 + t/4) at dim D0 + 4*(t%4) and receives V[K0 + j][D0 + t],
+// j = 0..3, i.e. a 4-key x 16-dim block transposed on the way out of LDS.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -60,33 +62,25 @@ struct KsaOps<KsaF16> {
     }
 };
 
-// low halves / high halves of two dwords -> one dword (lo16 from b, hi16 from a)
-__device__ __forceinline__ uint32_t ksa_pack_lo(uint32_t a, uint32_t b) {
-    return __builtin_amdgcn_perm(a, b, 0x05040100u);
-}
-__device__ __forceinline__ uint32_t ksa_pack_hi(uint32_t a, uint32_t b) {
-    return __builtin_amdgcn_perm(a, b, 0x07060302u);
-}
+typedef short ksa_short4 __attribute__((ext_vector_type(4)));
 
-// LDS position of key (4*kv4 .. 4*kv4+3) inside a V^T row
-__device__ __forceinline__ int ksa_vt_pos(int kv4) {
-    return 16 * (kv4 >> 2) + 8 * (kv4 & 1) + 4 * ((kv4 >> 1) & 1);
-}
-
-// Four rows x eight columns held as four 16-byte registers -> eight 8-byte
-// columns written to V^T rows d0 .. d0+7 at key position pos.
+// A operand of O^T += V^T P^T for k-step ks and 32-dim block db, from row-major V in LDS
+// (row stride VROW elements).  lq = lane % 32, lh = lane / 32.
 template <int VROW>
-__device__ __forceinline__ void ksa_store_vt(uint16_t* vt, int d0, int pos, const u32x4 (&r)[4]) {
-#pragma unroll
-    for (int w = 0; w < 4; ++w) {
-        u32x2 even, odd;
-        even[0] = ksa_pack_lo(r[1][w], r[0][w]);
-        even[1] = ksa_pack_lo(r[3][w], r[2][w]);
-        odd[0] = ksa_pack_hi(r[1][w], r[0][w]);
-        odd[1] = ksa_pack_hi(r[3][w], r[2][w]);
-        *reinterpret_cast<u32x2*>(vt + (d0 + 2 * w) * VROW + pos) = even;
-        *reinterpret_cast<u32x2*>(vt + (d0 + 2 * w + 1) * VROW + pos) = odd;
-    }
+__device__ __forceinline__ u32x4 ksa_read_vt_frag(const uint16_t* vs, int ks, int db, int lq, int lh) {
+    const int t = lq & 15;
+    const uint16_t* p = vs + (16 * ks + 4 * lh + (t >> 2)) * VROW + 32 * db + (lq & 16) + 4 * (t & 3);
+    typedef __attribute__((address_space(3))) ksa_short4* lds_ptr;
+    const ksa_short4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p));
+    const ksa_short4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p + 8 * VROW));
+    const u32x2 l2 = __builtin_bit_cast(u32x2, lo);
+    const u32x2 h2 = __builtin_bit_cast(u32x2, hi);
+    u32x4 r;
+    r[0] = l2[0];
+    r[1] = l2[1];
+    r[2] = h2[0];
+    r[3] = h2[1];
+    return r;
 }
 
 __device__ __forceinline__ float ksa_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
