@@ -22,6 +22,8 @@
 #include <hip/hip_runtime.h>
 #include <math.h>
 
+#include <type_traits>
+
 #include "ksa_api_internal.h"
 #include "ksa_mask.h"
 #include "ksa_tile.h"
@@ -58,6 +60,38 @@ constexpr int kThreads = 256;
 constexpr int kTileM = 128;
 constexpr int kTileN = 64;
 
+// Visible key set of one query row in key coordinates, fixed for the whole tile walk:
+//   [0, xa)   filtered by `a_sum_only` (in-line mode: summary columns only)
+//   [blo, bhi) filtered by `b_text`     (text rows: text columns only)
+struct RowVis {
+    int xa, blo, bhi;
+    bool b_text;
+};
+
+__device__ __forceinline__ RowVis ksa_row_vis(const KsaMask& mk, int q) {
+    const int B = mk.C + mk.S;
+    const int c = q / B, o = q % B;
+    RowVis r;
+    if (o >= mk.C) {  // summary row: own chunk, causal, every column kind
+        r.xa = 0;
+        r.blo = mk.P + c * B;
+        r.bhi = mk.P + q + 1;
+        r.b_text = false;
+        return r;
+    }
+    const int w0 = c > mk.W ? c - mk.W : 0;
+    r.b_text = true;
+    r.bhi = mk.P + q + 1;
+    if (mk.P > 0) {
+        r.xa = mk.skip_old ? 0 : w0 * mk.S;
+        r.blo = max(mk.P + w0 * B, r.xa);
+    } else {
+        r.xa = mk.skip_old ? 0 : w0 * B;
+        r.blo = w0 * B;
+    }
+    return r;
+}
+
 template <typename T, int D>
 __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillParams p) {
     using Ops = KsaOps<T>;
@@ -67,6 +101,8 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
     constexpr int VROW = D + 16;     // padded LDS row of V (stride = 8 banks mod 64)
     constexpr int CPR = D / 8;       // 16-byte chunks per K/V row
     constexpr int KLD = (kTileN * CPR) / kThreads;  // K (and V) loads per thread
+    constexpr int RSTEP = kThreads / CPR;           // row distance between a thread's loads
+    constexpr float kTau = 8.f;      // lazy rescale: exponents stay below 2^kTau
 
     __shared__ __attribute__((aligned(16))) uint16_t Ks[2][kTileN * KROW];
     __shared__ __attribute__((aligned(16))) uint16_t Vs[2][kTileN * VROW];
@@ -87,9 +123,11 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
     const int mt = p.M - 1 - rest / p.g;
     const int head = kvh * p.g + gi;
     const KsaMask mk = p.mk;
+    const bool prefix_mode = mk.P > 0;
 
     const int qrow = mt * kTileM + wave * 32 + lq;
     const int qrow_c = min(qrow, mk.Sq - 1);
+    const RowVis rv = ksa_row_vis(mk, qrow_c);
 
     // Q as B operand, resident in registers for the whole tile walk
     u32x4 qf[KS];
@@ -99,11 +137,18 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
         for (int s = 0; s < KS; ++s) qf[s] = *reinterpret_cast<const u32x4*>(qp + 16 * s);
     }
 
-    const uint16_t* kbase = p.k + bz * p.k_bs + kvh * p.k_hs;
-    const uint16_t* vbase = p.v + bz * p.v_bs + kvh * p.v_hs;
-    const uint16_t* kpbase = p.kprefix ? p.kprefix + bz * p.kp_bs + kvh * p.kp_hs : nullptr;
-    const uint16_t* vpbase = p.vprefix ? p.vprefix + bz * p.vp_bs + kvh * p.vp_hs : nullptr;
+    // K/V sources as uniform byte pointers + 32-bit per-thread byte offsets
+    const char* kmain = reinterpret_cast<const char*>(p.k + bz * p.k_bs + kvh * p.k_hs);
+    const char* vmain = reinterpret_cast<const char*>(p.v + bz * p.v_bs + kvh * p.v_hs);
+    const bool sep_prefix = p.kprefix != nullptr;
+    const char* kpre = sep_prefix ? reinterpret_cast<const char*>(p.kprefix + bz * p.kp_bs + kvh * p.kp_hs) : kmain;
+    const char* vpre = sep_prefix ? reinterpret_cast<const char*>(p.vprefix + bz * p.vp_bs + kvh * p.vp_hs) : vmain;
+    const uint32_t k_rb = (uint32_t)p.k_rs * 2u, v_rb = (uint32_t)p.v_rs * 2u;      // row bytes
+    const uint32_t kp_rb = sep_prefix ? (uint32_t)p.kp_rs * 2u : k_rb;
+    const uint32_t vp_rb = sep_prefix ? (uint32_t)p.vp_rs * 2u : v_rb;
     const int Bblk = mk.C + mk.S;
+    const int ld_row = tid / CPR;               // first tile row this thread loads
+    const uint32_t ld_col = (uint32_t)(tid % CPR) * 16u;
 
     const int npart = p.mask_cnt[mt];
     const int ntiles = npart + p.full_cnt[mt];
@@ -113,68 +158,108 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
     u32x4 kreg[KLD];
     u32x4 vreg[KLD];
 
-    auto row_ptrs = [&](int kv, const uint16_t*& kr, const uint16_t*& vr) {
-        kv = min(kv, mk.Sk - 1);
-        if (kv < mk.P) {
-            if (kpbase) {
-                kr = kpbase + (int64_t)kv * p.kp_rs;
-                vr = vpbase + (int64_t)kv * p.vp_rs;
-            } else {  // prefix row j lives at in-line row (j/S)*B + C + j%S
-                const int r = (kv / mk.S) * Bblk + mk.C + (kv % mk.S);
-                kr = kbase + (int64_t)r * p.k_rs;
-                vr = vbase + (int64_t)r * p.v_rs;
-            }
-        } else {
-            kr = kbase + (int64_t)(kv - mk.P) * p.k_rs;
-            vr = vbase + (int64_t)(kv - mk.P) * p.v_rs;
-        }
-    };
+    // in-line row that holds prefix row j (periodic summary layout)
+    auto inline_row = [&](int j) { return (j / mk.S) * Bblk + mk.C + (j % mk.S); };
 
     auto load_tile = [&](int n) {
         const int n0 = n * kTileN;
+        if (n0 >= mk.P && n0 + kTileN <= mk.Sk) {  // tile entirely in the in-line region
+            const uint32_t r0 = (uint32_t)(n0 - mk.P + ld_row);
 #pragma unroll
-        for (int i = 0; i < KLD; ++i) {
-            const int u = tid + kThreads * i;
-            const int row = u / CPR, c = u % CPR;
-            const uint16_t *kr, *vr;
-            row_ptrs(n0 + row, kr, vr);
-            kreg[i] = *reinterpret_cast<const u32x4*>(kr + 8 * c);
-            vreg[i] = *reinterpret_cast<const u32x4*>(vr + 8 * c);
+            for (int i = 0; i < KLD; ++i) {
+                kreg[i] = *reinterpret_cast<const u32x4*>(kmain + ((r0 + RSTEP * i) * k_rb + ld_col));
+                vreg[i] = *reinterpret_cast<const u32x4*>(vmain + ((r0 + RSTEP * i) * v_rb + ld_col));
+            }
+        } else if (n0 + kTileN <= mk.P) {  // tile entirely in the summary prefix
+#pragma unroll
+            for (int i = 0; i < KLD; ++i) {
+                const int j = n0 + ld_row + RSTEP * i;
+                const uint32_t r = (uint32_t)(sep_prefix ? j : inline_row(j));
+                kreg[i] = *reinterpret_cast<const u32x4*>(kpre + (r * kp_rb + ld_col));
+                vreg[i] = *reinterpret_cast<const u32x4*>(vpre + (r * vp_rb + ld_col));
+            }
+        } else {  // straddles the prefix end or the end of the key axis
+#pragma unroll
+            for (int i = 0; i < KLD; ++i) {
+                const int kv = min(n0 + ld_row + RSTEP * i, mk.Sk - 1);
+                const bool pre = kv < mk.P;
+                const uint32_t r = (uint32_t)(pre ? (sep_prefix ? kv : inline_row(kv)) : kv - mk.P);
+                const char* kb = pre ? kpre : kmain;
+                const char* vb = pre ? vpre : vmain;
+                kreg[i] = *reinterpret_cast<const u32x4*>(kb + (r * (pre ? kp_rb : k_rb) + ld_col));
+                vreg[i] = *reinterpret_cast<const u32x4*>(vb + (r * (pre ? vp_rb : v_rb) + ld_col));
+            }
         }
     };
 
     auto store_tile = [&](int buf) {
 #pragma unroll
         for (int i = 0; i < KLD; ++i) {
-            const int u = tid + kThreads * i;
-            const int row = u / CPR, c = u % CPR;
-            *reinterpret_cast<u32x4*>(&Ks[buf][row * KROW + 8 * c]) = kreg[i];
-            *reinterpret_cast<u32x4*>(&Vs[buf][row * VROW + 8 * c]) = vreg[i];
+            const int row = ld_row + RSTEP * i;
+            *reinterpret_cast<u32x4*>(&Ks[buf][row * KROW + 8 * (tid % CPR)]) = kreg[i];
+            *reinterpret_cast<u32x4*>(&Vs[buf][row * VROW + 8 * (tid % CPR)]) = vreg[i];
         }
     };
 
-    auto tile_at = [&](int i) { return i < npart ? plist[i] : flist[i - npart]; };
+    // Walk order.  Phase A: tiles that need no per-element mask -- the leading partial
+    // tiles that lie below every text row's old-summary bound (there a row is visible
+    // as a whole iff it is a text row) and the full tiles.  Phase B: the remaining
+    // partial tiles (and a full tile cut by the end of the key axis), masked per element.
+    // The split is uniform for the workgroup so that all waves walk the same sequence.
+    int nquick = 0;
+    {
+        const int q_first = mt * kTileM;
+        const int c_first = q_first / Bblk;
+        const int w_first = c_first > mk.W ? c_first - mk.W : 0;
+        // every text row of the tile has xa >= w_first * S and blo >= P + w_first * B >= thr
+        const int thr = (prefix_mode && !mk.skip_old) ? min(w_first * mk.S, mk.P) : 0;
+        const int nlim = thr / kTileN;  // tiles n < nlim end at or below thr
+        int lo = 0, hi = npart;         // first index with plist[i] >= nlim
+        while (lo < hi) {
+            const int mid = (lo + hi) >> 1;
+            if (plist[mid] < nlim) lo = mid + 1; else hi = mid;
+        }
+        nquick = lo;
+    }
+    const int nfull = p.full_cnt[mt];
+    const bool last_full_cut = nfull > 0 && (flist[nfull - 1] + 1) * kTileN > mk.Sk;
+    const int nfull_a = nfull - (last_full_cut ? 1 : 0);
+    const int n_a = nquick + nfull_a;
+    auto tile_at = [&](int i) {
+        if (i < nquick) return plist[i];
+        if (i < n_a) return flist[i - nquick];
+        const int j = i - n_a + nquick;
+        return j < npart ? plist[j] : flist[nfull - 1];
+    };
+    const bool lane_is_text = rv.b_text;
+    // The walk order is kept in registers, 64 entries at a time (lane i holds entry
+    // base + i), so the loop never waits on a dependent index load.
+    auto seq_chunk = [&](int base) { return base + lane < ntiles ? tile_at(base + lane) : 0; };
+    int seq_cur = seq_chunk(0);
+    int seq_nxt = seq_chunk(64);
 
     floatx16 oacc[DB];
 #pragma unroll
     for (int b = 0; b < DB; ++b)
 #pragma unroll
         for (int i = 0; i < 16; ++i) oacc[b][i] = 0.f;
-    float m_run = -INFINITY;
-    float l_run = 0.f;
+    float m_ref = -INFINITY;  // reference maximum of the exponents (raw score units)
+    float l_run = 0.f;        // this lane's half of the row sum
     const float c2 = p.scale_log2;
 
-    if (ntiles > 0) load_tile(tile_at(0));
-
-    for (int it = 0; it < ntiles; ++it) {
+    // One tile: scores, (optional) per-element mask, soft-max update, second product.
+    auto tile_body = [&](auto general_tag, int it, bool row_vis) {
+        constexpr bool kGeneral = decltype(general_tag)::value;
         const int buf = it & 1;
-        const int n = tile_at(it);
-        const int n0 = n * kTileN;
+        const int n0 = __builtin_amdgcn_readlane(seq_cur, it & 63) * kTileN;
         store_tile(buf);
         __syncthreads();
-        if (it + 1 < ntiles) load_tile(tile_at(it + 1));
+        if (it + 1 < ntiles) {
+            const int nn = ((it + 1) & 63) ? __builtin_amdgcn_readlane(seq_cur, (it + 1) & 63)
+                                           : __builtin_amdgcn_readlane(seq_nxt, 0);
+            load_tile(nn);
+        }
 
-        // ---- S^T = K Q^T ----
         floatx16 sacc[2];
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
@@ -190,41 +275,46 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
             }
         }
 
-        // ---- mask ----
-        bool row_vis = true;
-        const bool need_mask = (it < npart) || (n0 + kTileN > mk.Sk);
-        if (need_mask) {
-            uint64_t text, valid;
-            ksa_tile_column_bits(mk, n0, lane, text, valid);
-            const uint64_t bits = ksa_row_bits(mk, qrow_c, n0, text, valid);
-            const bool uniform = __all(bits == 0ull || bits == ~0ull);
-            if (uniform) {
-                row_vis = bits != 0ull;
-            } else {
-                const uint64_t sh = bits >> (4 * lh);
-                const uint32_t w0 = (uint32_t)sh, w1 = (uint32_t)(sh >> 32);
+        if constexpr (kGeneral) {  // 64-bit visibility word per row
+            const int kv = n0 + lane;
+            const int rel = kv - mk.P;
+            const bool in = kv < mk.Sk;
+            const uint64_t valid = __ballot(in);
+            const uint64_t text = __ballot(in && rel >= 0 && (rel % Bblk) < mk.C);
+            const uint64_t fa = prefix_mode ? valid : (valid & ~text);
+            const uint64_t fb = rv.b_text ? text : valid;
+            const uint64_t bits = (ksa_range_bits(-n0, rv.xa - n0) & fa) |
+                                  (ksa_range_bits(rv.blo - n0, rv.bhi - n0) & fb);
+            const uint64_t sh = bits >> (4 * lh);
+            const uint32_t w0 = (uint32_t)sh, w1 = (uint32_t)(sh >> 32);
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const uint32_t bit = 1u << (8 * (i / 4) + (i % 4));
-                    sacc[0][i] = (w0 & bit) ? sacc[0][i] : -INFINITY;
-                    sacc[1][i] = (w1 & bit) ? sacc[1][i] : -INFINITY;
-                }
+            for (int i = 0; i < 16; ++i) {
+                const uint32_t bit = 1u << (8 * (i / 4) + (i % 4));
+                sacc[0][i] = (w0 & bit) ? sacc[0][i] : -INFINITY;
+                sacc[1][i] = (w1 & bit) ? sacc[1][i] : -INFINITY;
             }
         }
 
-        // ---- online soft-max (one query row per lane pair l, l^32) ----
-        float mloc = -INFINITY;
+        float mloc = fmaxf(sacc[0][0], sacc[1][0]);
 #pragma unroll
-        for (int i = 0; i < 16; ++i) mloc = fmaxf(mloc, fmaxf(sacc[0][i], sacc[1][i]));
+        for (int i = 1; i < 16; ++i) mloc = fmaxf(mloc, fmaxf(sacc[0][i], sacc[1][i]));
         if (!row_vis) mloc = -INFINITY;
-        mloc = fmaxf(mloc, ksa_xor32(mloc));
-        const float m_new = fmaxf(m_run, mloc);
+        mloc = ksa_pair_max(mloc);
+        // lazy rescale: move the reference only when the row maximum outgrows it by 2^kTau
+        const bool bump = (mloc - m_ref) * c2 > kTau || m_ref == -INFINITY;
+        const float m_new = bump ? mloc : m_ref;
         const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = ksa_exp2((m_run - m_safe) * c2);
+        if (__any(bump && mloc != -INFINITY)) {
+            const float alpha = ksa_exp2((m_ref - m_safe) * c2);
+            l_run *= alpha;
+#pragma unroll
+            for (int b = 0; b < DB; ++b)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) oacc[b][i] *= alpha;
+        }
+        m_ref = m_new;
         const float mc = row_vis ? m_safe * c2 : INFINITY;
-        m_run = m_new;
 
-        float rowsum = 0.f;
         u32x4 pf[4];
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
@@ -232,19 +322,10 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
             for (int i = 0; i < 16; i += 2) {
                 const float p0 = ksa_exp2(fmaf(sacc[kb][i], c2, -mc));
                 const float p1 = ksa_exp2(fmaf(sacc[kb][i + 1], c2, -mc));
-                rowsum += p0 + p1;
-                pf[kb * 2 + i / 8][(i % 8) / 2] = Ops::pack2(p0, p1);
+                const uint32_t pk = Ops::pack2(p0, p1);
+                l_run = Ops::sum2(pk, l_run);
+                pf[kb * 2 + i / 8][(i % 8) / 2] = pk;
             }
-        l_run = l_run * alpha + rowsum;
-
-        if (__any(alpha != 1.f)) {
-#pragma unroll
-            for (int b = 0; b < DB; ++b)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) oacc[b][i] *= alpha;
-        }
-
-        // ---- O^T += V^T P^T ----
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
 #pragma unroll
@@ -253,10 +334,27 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
                 oacc[b] = Ops::mfma(a, pf[ks], oacc[b]);
             }
         }
+    };
+
+    if (ntiles > 0) load_tile(__builtin_amdgcn_readlane(seq_cur, 0));
+    auto advance = [&](int it) {  // after tile `it`: roll the index chunk every 64 tiles
+        if ((it & 63) == 63) {
+            seq_cur = seq_nxt;
+            seq_nxt = seq_chunk(it + 1 + 64);
+        }
+    };
+    int it = 0;
+    for (; it < n_a; ++it) {
+        tile_body(std::false_type{}, it, it < nquick ? lane_is_text : true);
+        advance(it);
+    }
+    for (; it < ntiles; ++it) {
+        tile_body(std::true_type{}, it, true);
+        advance(it);
     }
 
     // ---- epilogue ----
-    const float l_tot = l_run + ksa_xor32(l_run);
+    const float l_tot = ksa_pair_sum(l_run);
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
     if (qrow < mk.Sq) {
         uint16_t* op = p.out + bz * p.o_bs + (int64_t)qrow * p.o_rs + head * p.o_hs;
@@ -271,7 +369,7 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
             }
         if (p.lse && lh == 0)
             p.lse[bz * p.lse_bs + head * p.lse_hs + qrow] =
-                l_tot > 0.f ? m_run * p.scale + logf(l_tot) : -INFINITY;
+                l_tot > 0.f ? m_ref * p.scale + logf(l_tot) : -INFINITY;
     }
 }
 
@@ -303,6 +401,12 @@ extern "C" int ksa_prefill_fwd(const void* q, const void* k, const void* v, cons
     if (batch <= 0 || Sq <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0) return KSA_ERR_INVALID;
     if (C <= 0 || S <= 0 || W < 0 || P < 0) return KSA_ERR_INVALID;
     if ((int64_t)Sq + P >= (1ll << 30)) return KSA_ERR_INVALID;
+    // K/V rows are addressed with 32-bit byte offsets inside one (batch, head) slice
+    if ((int64_t)Sq * k_strides[1] * 2 >= (1ll << 32) || (int64_t)Sq * v_strides[1] * 2 >= (1ll << 32))
+        return KSA_ERR_INVALID;
+    if (kprefix && ((int64_t)P * kprefix_strides[1] * 2 >= (1ll << 32) ||
+                    (int64_t)P * vprefix_strides[1] * 2 >= (1ll << 32)))
+        return KSA_ERR_INVALID;
     if (dtype != KSA_DTYPE_BF16 && dtype != KSA_DTYPE_F16) return KSA_ERR_UNSUPPORTED;
     const int Sk = Sq + P;
     const int N = (Sk + kTileN - 1) / kTileN;

@@ -46,6 +46,13 @@ struct KsaOps<KsaBf16> {
         v[1] = (__bf16)hi;
         return __builtin_bit_cast(uint32_t, v);
     }
+    // acc + lo + hi of a packed pair (as rounded to 16 bit)
+    static __device__ __forceinline__ float sum2(uint32_t pk, float acc) {
+        bf16x2 one;
+        one[0] = (__bf16)1.0f;
+        one[1] = (__bf16)1.0f;
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pk), one, acc, false);
+    }
 };
 
 template <>
@@ -59,6 +66,12 @@ struct KsaOps<KsaF16> {
         v[0] = (_Float16)lo;
         v[1] = (_Float16)hi;
         return __builtin_bit_cast(uint32_t, v);
+    }
+    static __device__ __forceinline__ float sum2(uint32_t pk, float acc) {
+        f16x2 one;
+        one[0] = (_Float16)1.0f;
+        one[1] = (_Float16)1.0f;
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, pk), one, acc, false);
     }
 };
 
@@ -86,6 +99,19 @@ __device__ __forceinline__ u32x4 ksa_read_vt_frag(const uint16_t* vs, int ks, in
 __device__ __forceinline__ float ksa_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 __device__ __forceinline__ float ksa_xor32(float x) { return __shfl_xor(x, 32); }
+
+// Reductions over the lane pair (l, l ^ 32) with v_permlane32_swap: after the swap one
+// result holds the lower half's value and the other the upper half's value in every lane.
+__device__ __forceinline__ float ksa_pair_max(float x) {
+    const uint32_t u = __builtin_bit_cast(uint32_t, x);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return fmaxf(__builtin_bit_cast(float, (uint32_t)r[0]), __builtin_bit_cast(float, (uint32_t)r[1]));
+}
+__device__ __forceinline__ float ksa_pair_sum(float x) {
+    const uint32_t u = __builtin_bit_cast(uint32_t, x);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return __builtin_bit_cast(float, (uint32_t)r[0]) + __builtin_bit_cast(float, (uint32_t)r[1]);
+}
 
 // fence that orders this wave's LDS writes before its later LDS reads (and the
 // reverse) without involving the other waves of the workgroup
