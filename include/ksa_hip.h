@@ -56,22 +56,23 @@ int ksa_block_index(int Sq, int Sk, int C, int S, int W, int P, int skip_old, in
  * Replaces whl-sa:summary_attn/interface.py:271-289 (summary_attn_func) ->
  * :70-91 (SummaryAttnFunc.forward) -> whl-fa:flash_attn/cute/interface.py:85-534
  * (_flash_attn_fwd with mask_mod + block_sparse_tensors, tiles 128 x 64).
- *   q   [batch, Sq, Hq,  D]   strides {batch, row, head}
- *   k,v [batch, Sq, Hkv, D]   in-line keys / values
- *   kprefix, vprefix: the P summary rows as separate tensors [batch, P, Hkv, D], or NULL:
- *       then prefix row j is read in place from in-line row (j/S)*(C+S) + C + j%S
- *       (what `k[:, summary_pos]` gathers when summary_pos is the periodic pattern).
+ *   q   [batch, Sq, Hq, D]        strides {batch, row, head}
+ *   k,v [batch, rows, Hkv, D]     one stride triple for both (kv_strides)
+ *       phys_prefix == 0: rows = Sq in-line keys; prefix row j (j < P) is read in place
+ *           from in-line row (j/S)*(C+S) + C + j%S -- what `k[:, summary_pos]` gathers
+ *           when summary_pos is the periodic pattern; nothing is concatenated.
+ *       phys_prefix != 0: rows = P + Sq, the layout the reference builds with
+ *           torch.cat((k[:, summary_pos], k), dim=1).
+ *       rows * row stride * 2 bytes must stay below 4 GiB.
  *   out [batch, Sq, Hq, D]; lse fp32 [batch, Hq, Sq] (natural log) or NULL.
  *   mask_cnt .. full_idx: output of ksa_block_index(Sq, Sq+P, ..., 128, 64), idx_stride = N.
  *   scale: soft-max scale (the reference uses head_dim^-0.5). */
-int ksa_prefill_fwd(const void* q, const void* k, const void* v, const void* kprefix,
-                    const void* vprefix, void* out, float* lse, int batch, int Sq, int Hq, int Hkv,
-                    int D, int dtype, const int64_t* q_strides, const int64_t* k_strides,
-                    const int64_t* v_strides, const int64_t* kprefix_strides,
-                    const int64_t* vprefix_strides, const int64_t* out_strides, int C, int S, int W,
-                    int P, int skip_old, const int32_t* mask_cnt, const int32_t* mask_idx,
-                    const int32_t* full_cnt, const int32_t* full_idx, int idx_stride, float scale,
-                    void* stream);
+int ksa_prefill_fwd(const void* q, const void* k, const void* v, void* out, float* lse, int batch,
+                    int Sq, int Hq, int Hkv, int D, int dtype, const int64_t* q_strides,
+                    const int64_t* kv_strides, const int64_t* out_strides, int C, int S, int W,
+                    int P, int skip_old, int phys_prefix, const int32_t* mask_cnt,
+                    const int32_t* mask_idx, const int32_t* full_cnt, const int32_t* full_idx,
+                    int idx_stride, float scale, void* stream);
 
 /* Decode attention over the ring-buffer slice.
  * Replaces HF:591-612 (_sdpa_attention_forward, incl. repeat_kv :557-566) applied to the

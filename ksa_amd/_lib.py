@@ -21,7 +21,7 @@ _SIGNATURES = {
     "ksa_error_string": (ctypes.c_char_p, [_int]),
     "ksa_device_cu_count": (_int, []),
     "ksa_block_index": (_int, [_int] * 9 + [_vp] * 4 + [_vp]),
-    "ksa_prefill_fwd": (_int, [_vp] * 7 + [_int] * 6 + [_i64p] * 6 + [_int] * 5 + [_vp] * 4
+    "ksa_prefill_fwd": (_int, [_vp] * 5 + [_int] * 6 + [_i64p] * 3 + [_int] * 6 + [_vp] * 4
                         + [_int, ctypes.c_float, _vp]),
     "ksa_decode_workspace_bytes": (ctypes.c_size_t, [_int] * 6),
     "ksa_decode_auto_splits": (_int, [_int] * 3),

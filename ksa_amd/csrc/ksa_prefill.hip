@@ -11,14 +11,20 @@
 //
 // One workgroup (4 waves) owns a 128-row query tile of one query head; wave w owns
 // rows 32w .. 32w+31.  It walks the tile's non-empty key tiles (64 keys each) taken
-// from the block index, staging K and V row-major in LDS (two buffers); V is transposed
-// on the way out of LDS by ds_read_b64_tr_b16, see ksa_tile.h for the operand layouts.  The summary prefix of the key axis is
-// read in place from the in-line summary rows (or from a separate prefix buffer),
-// never concatenated.
+// from the block index, staging K and V row-major in LDS (two buffers each); V is
+// transposed on the way out of LDS by ds_read_b64_tr_b16 (operand layouts: ksa_tile.h).
+// The summary prefix of the key axis is read in place from the in-line summary rows
+// (or, with `phys_prefix`, from the first P rows of K/V), never concatenated.
 //
-// Partial tiles are masked from a 64-bit visibility word per query row; when every
-// row of the wave is all-or-nothing in the tile (the common case: summary rows do
-// not see old summaries, text rows see all of them) no per-element work is done.
+// The loop is software-pipelined: the score MFMAs of tile i+1 are issued before the
+// soft-max of tile i so that matrix and vector work of one wave overlap; K therefore
+// runs one tile ahead of V through LDS.
+//
+// Masking.  The walk has two phases that are uniform for the workgroup.  Phase A holds
+// the tiles that need no per-element mask: the leading partial tiles below every text
+// row's old-summary bound (there a row is visible as a whole iff it is a text row) and
+// the full tiles.  Phase B holds the remaining partial tiles, masked per element from a
+// 64-bit visibility word per query row.
 #include <hip/hip_runtime.h>
 #include <math.h>
 
@@ -32,10 +38,8 @@ namespace {
 
 struct PrefillParams {
     const uint16_t* q;
-    const uint16_t* k;        // in-line keys   [Sq rows]
+    const uint16_t* k;
     const uint16_t* v;
-    const uint16_t* kprefix;  // separate prefix rows [P rows] or null (read in place)
-    const uint16_t* vprefix;
     uint16_t* out;
     float* lse;  // may be null
     const int32_t* mask_cnt;
@@ -44,11 +48,9 @@ struct PrefillParams {
     const int32_t* full_idx;
     int idx_stride;  // N
     int M, Hq, Hkv, g;
-    int64_t q_bs, q_rs, q_hs;  // element strides: batch, row, head
-    int64_t k_bs, k_rs, k_hs;
-    int64_t v_bs, v_rs, v_hs;
-    int64_t kp_bs, kp_rs, kp_hs;
-    int64_t vp_bs, vp_rs, vp_hs;
+    int phys_prefix;            // K/V rows are [P prefix rows | Sq in-line rows]
+    int64_t q_bs, q_rs, q_hs;   // element strides: batch, row, head
+    int64_t kv_bs, kv_rs, kv_hs;
     int64_t o_bs, o_rs, o_hs;
     int64_t lse_bs, lse_hs;
     KsaMask mk;
@@ -61,8 +63,8 @@ constexpr int kTileM = 128;
 constexpr int kTileN = 64;
 
 // Visible key set of one query row in key coordinates, fixed for the whole tile walk:
-//   [0, xa)   filtered by `a_sum_only` (in-line mode: summary columns only)
-//   [blo, bhi) filtered by `b_text`     (text rows: text columns only)
+//   [0, xa)    (in-line mode: summary columns only)
+//   [blo, bhi) (text rows: text columns only)
 struct RowVis {
     int xa, blo, bhi;
     bool b_text;
@@ -124,6 +126,8 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
     const int head = kvh * p.g + gi;
     const KsaMask mk = p.mk;
     const bool prefix_mode = mk.P > 0;
+    const bool phys = p.phys_prefix != 0;
+    const int Bblk = mk.C + mk.S;
 
     const int qrow = mt * kTileM + wave * 32 + lq;
     const int qrow_c = min(qrow, mk.Sq - 1);
@@ -137,81 +141,86 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
         for (int s = 0; s < KS; ++s) qf[s] = *reinterpret_cast<const u32x4*>(qp + 16 * s);
     }
 
-    // K/V sources as uniform byte pointers + 32-bit per-thread byte offsets
-    const char* kmain = reinterpret_cast<const char*>(p.k + bz * p.k_bs + kvh * p.k_hs);
-    const char* vmain = reinterpret_cast<const char*>(p.v + bz * p.v_bs + kvh * p.v_hs);
-    const bool sep_prefix = p.kprefix != nullptr;
-    const char* kpre = sep_prefix ? reinterpret_cast<const char*>(p.kprefix + bz * p.kp_bs + kvh * p.kp_hs) : kmain;
-    const char* vpre = sep_prefix ? reinterpret_cast<const char*>(p.vprefix + bz * p.vp_bs + kvh * p.vp_hs) : vmain;
-    const uint32_t k_rb = (uint32_t)p.k_rs * 2u, v_rb = (uint32_t)p.v_rs * 2u;      // row bytes
-    const uint32_t kp_rb = sep_prefix ? (uint32_t)p.kp_rs * 2u : k_rb;
-    const uint32_t vp_rb = sep_prefix ? (uint32_t)p.vp_rs * 2u : v_rb;
-    const int Bblk = mk.C + mk.S;
-    const int ld_row = tid / CPR;               // first tile row this thread loads
+    // ---- K/V addressing: uniform base + uniform tile offset + 32-bit thread offset ----
+    const char* kbase = reinterpret_cast<const char*>(p.k + bz * p.kv_bs + kvh * p.kv_hs);
+    const char* vbase = reinterpret_cast<const char*>(p.v + bz * p.kv_bs + kvh * p.kv_hs);
+    const uint32_t rb = (uint32_t)p.kv_rs * 2u;  // row pitch in bytes
+    const int ld_row = tid / CPR;                // first tile row this thread loads
     const uint32_t ld_col = (uint32_t)(tid % CPR) * 16u;
+    const uint32_t thr_main = (uint32_t)ld_row * rb + ld_col;
+    // in-place prefix: prefix row j lives at in-line row (j / S) * B + C + j % S; when S
+    // divides the per-thread row step the rows of one thread differ by a uniform amount
+    const bool s_fast = !phys && (RSTEP % mk.S == 0);
+    const uint32_t thr_pre =
+        s_fast ? (uint32_t)((ld_row / mk.S) * Bblk + mk.C + ld_row % mk.S) * rb + ld_col : 0u;
+    const uint32_t step_main = RSTEP * rb;
+    const uint32_t step_pre = s_fast ? (uint32_t)(RSTEP / mk.S) * Bblk * rb : 0u;
 
-    const int npart = p.mask_cnt[mt];
-    const int ntiles = npart + p.full_cnt[mt];
-    const int32_t* plist = p.mask_idx + (int64_t)mt * p.idx_stride;
-    const int32_t* flist = p.full_idx + (int64_t)mt * p.idx_stride;
+    auto src_row = [&](int kv) -> uint32_t {  // generic key column -> K/V row
+        kv = min(kv, mk.Sk - 1);
+        if (phys || kv >= mk.P) return (uint32_t)(phys ? kv : kv - mk.P);
+        return (uint32_t)((kv / mk.S) * Bblk + mk.C + kv % mk.S);
+    };
+
+    // tile -> (uniform byte offset, uniform per-load step, per-thread byte offsets)
+    auto tile_src = [&](int n0, uint32_t& ubase, uint32_t& ustep, uint32_t (&voff)[KLD]) {
+        const bool in_main = (phys || n0 >= mk.P) && n0 + kTileN <= mk.Sk;
+        if (in_main) {
+            ubase = (uint32_t)(phys ? n0 : n0 - mk.P) * rb;
+            ustep = step_main;
+#pragma unroll
+            for (int i = 0; i < KLD; ++i) voff[i] = thr_main;
+        } else if (s_fast && n0 + kTileN <= mk.P) {
+            ubase = (uint32_t)(n0 / mk.S) * Bblk * rb;
+            ustep = step_pre;
+#pragma unroll
+            for (int i = 0; i < KLD; ++i) voff[i] = thr_pre;
+        } else {
+            ubase = 0;
+            ustep = 0;
+#pragma unroll
+            for (int i = 0; i < KLD; ++i) voff[i] = src_row(n0 + ld_row + RSTEP * i) * rb + ld_col;
+        }
+    };
 
     u32x4 kreg[KLD];
     u32x4 vreg[KLD];
-
-    // in-line row that holds prefix row j (periodic summary layout)
-    auto inline_row = [&](int j) { return (j / mk.S) * Bblk + mk.C + (j % mk.S); };
-
-    auto load_tile = [&](int n) {
-        const int n0 = n * kTileN;
-        if (n0 >= mk.P && n0 + kTileN <= mk.Sk) {  // tile entirely in the in-line region
-            const uint32_t r0 = (uint32_t)(n0 - mk.P + ld_row);
+    auto load_k = [&](int n) {
+        uint32_t ub, us, vo[KLD];
+        tile_src(n * kTileN, ub, us, vo);
 #pragma unroll
-            for (int i = 0; i < KLD; ++i) {
-                kreg[i] = *reinterpret_cast<const u32x4*>(kmain + ((r0 + RSTEP * i) * k_rb + ld_col));
-                vreg[i] = *reinterpret_cast<const u32x4*>(vmain + ((r0 + RSTEP * i) * v_rb + ld_col));
-            }
-        } else if (n0 + kTileN <= mk.P) {  // tile entirely in the summary prefix
+        for (int i = 0; i < KLD; ++i)
+            kreg[i] = *reinterpret_cast<const u32x4*>(kbase + (ub + us * i) + vo[i]);
+    };
+    auto load_v = [&](int n) {
+        uint32_t ub, us, vo[KLD];
+        tile_src(n * kTileN, ub, us, vo);
 #pragma unroll
-            for (int i = 0; i < KLD; ++i) {
-                const int j = n0 + ld_row + RSTEP * i;
-                const uint32_t r = (uint32_t)(sep_prefix ? j : inline_row(j));
-                kreg[i] = *reinterpret_cast<const u32x4*>(kpre + (r * kp_rb + ld_col));
-                vreg[i] = *reinterpret_cast<const u32x4*>(vpre + (r * vp_rb + ld_col));
-            }
-        } else {  // straddles the prefix end or the end of the key axis
+        for (int i = 0; i < KLD; ++i)
+            vreg[i] = *reinterpret_cast<const u32x4*>(vbase + (ub + us * i) + vo[i]);
+    };
+    auto store_k = [&](int buf) {
 #pragma unroll
-            for (int i = 0; i < KLD; ++i) {
-                const int kv = min(n0 + ld_row + RSTEP * i, mk.Sk - 1);
-                const bool pre = kv < mk.P;
-                const uint32_t r = (uint32_t)(pre ? (sep_prefix ? kv : inline_row(kv)) : kv - mk.P);
-                const char* kb = pre ? kpre : kmain;
-                const char* vb = pre ? vpre : vmain;
-                kreg[i] = *reinterpret_cast<const u32x4*>(kb + (r * (pre ? kp_rb : k_rb) + ld_col));
-                vreg[i] = *reinterpret_cast<const u32x4*>(vb + (r * (pre ? vp_rb : v_rb) + ld_col));
-            }
-        }
+        for (int i = 0; i < KLD; ++i)
+            *reinterpret_cast<u32x4*>(&Ks[buf][(ld_row + RSTEP * i) * KROW + 8 * (tid % CPR)]) = kreg[i];
+    };
+    auto store_v = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < KLD; ++i)
+            *reinterpret_cast<u32x4*>(&Vs[buf][(ld_row + RSTEP * i) * VROW + 8 * (tid % CPR)]) = vreg[i];
     };
 
-    auto store_tile = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < KLD; ++i) {
-            const int row = ld_row + RSTEP * i;
-            *reinterpret_cast<u32x4*>(&Ks[buf][row * KROW + 8 * (tid % CPR)]) = kreg[i];
-            *reinterpret_cast<u32x4*>(&Vs[buf][row * VROW + 8 * (tid % CPR)]) = vreg[i];
-        }
-    };
-
-    // Walk order.  Phase A: tiles that need no per-element mask -- the leading partial
-    // tiles that lie below every text row's old-summary bound (there a row is visible
-    // as a whole iff it is a text row) and the full tiles.  Phase B: the remaining
-    // partial tiles (and a full tile cut by the end of the key axis), masked per element.
-    // The split is uniform for the workgroup so that all waves walk the same sequence.
+    // ---- walk order ----
+    const int npart = p.mask_cnt[mt];
+    const int nfull = p.full_cnt[mt];
+    const int ntiles = npart + nfull;
+    const int32_t* plist = p.mask_idx + (int64_t)mt * p.idx_stride;
+    const int32_t* flist = p.full_idx + (int64_t)mt * p.idx_stride;
     int nquick = 0;
     {
-        const int q_first = mt * kTileM;
-        const int c_first = q_first / Bblk;
+        const int c_first = (mt * kTileM) / Bblk;
         const int w_first = c_first > mk.W ? c_first - mk.W : 0;
-        // every text row of the tile has xa >= w_first * S and blo >= P + w_first * B >= thr
+        // every text row of the tile has xa >= w_first * S and blo >= P >= thr
         const int thr = (prefix_mode && !mk.skip_old) ? min(w_first * mk.S, mk.P) : 0;
         const int nlim = thr / kTileN;  // tiles n < nlim end at or below thr
         int lo = 0, hi = npart;         // first index with plist[i] >= nlim
@@ -221,7 +230,6 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
         }
         nquick = lo;
     }
-    const int nfull = p.full_cnt[mt];
     const bool last_full_cut = nfull > 0 && (flist[nfull - 1] + 1) * kTileN > mk.Sk;
     const int nfull_a = nfull - (last_full_cut ? 1 : 0);
     const int n_a = nquick + nfull_a;
@@ -231,12 +239,16 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
         const int j = i - n_a + nquick;
         return j < npart ? plist[j] : flist[nfull - 1];
     };
-    const bool lane_is_text = rv.b_text;
-    // The walk order is kept in registers, 64 entries at a time (lane i holds entry
-    // base + i), so the loop never waits on a dependent index load.
+    // The order is kept in registers, 64 entries at a time (lane i holds entry base + i),
+    // so the loop never waits on a dependent index load.
     auto seq_chunk = [&](int base) { return base + lane < ntiles ? tile_at(base + lane) : 0; };
     int seq_cur = seq_chunk(0);
     int seq_nxt = seq_chunk(64);
+    auto seq = [&](int i, int it) {  // entry i in {it, it+1, it+2} while processing tile it
+        const int c = (i >> 6) - (it >> 6);
+        return c == 0 ? __builtin_amdgcn_readlane(seq_cur, i & 63)
+                      : __builtin_amdgcn_readlane(seq_nxt, i & 63);
+    };
 
     floatx16 oacc[DB];
 #pragma unroll
@@ -247,20 +259,7 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
     float l_run = 0.f;        // this lane's half of the row sum
     const float c2 = p.scale_log2;
 
-    // One tile: scores, (optional) per-element mask, soft-max update, second product.
-    auto tile_body = [&](auto general_tag, int it, bool row_vis) {
-        constexpr bool kGeneral = decltype(general_tag)::value;
-        const int buf = it & 1;
-        const int n0 = __builtin_amdgcn_readlane(seq_cur, it & 63) * kTileN;
-        store_tile(buf);
-        __syncthreads();
-        if (it + 1 < ntiles) {
-            const int nn = ((it + 1) & 63) ? __builtin_amdgcn_readlane(seq_cur, (it + 1) & 63)
-                                           : __builtin_amdgcn_readlane(seq_nxt, 0);
-            load_tile(nn);
-        }
-
-        floatx16 sacc[2];
+    auto scores = [&](floatx16 (&sacc)[2], int buf) {  // S^T = K Q^T for the tile in Ks[buf]
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
@@ -273,6 +272,22 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
                     &Ks[buf][(kb * 32 + lq) * KROW + 16 * s + 8 * lh]);
                 sacc[kb] = Ops::mfma(a, qf[s], sacc[kb]);
             }
+        }
+    };
+
+    // One pipeline step for tile `it`: its scores are in `scur`; the scores of tile it+1
+    // are produced into `snext`.  On entry the registers hold K(it+1) and V(it).
+    auto step = [&](auto general_tag, int it, floatx16 (&scur)[2], floatx16 (&snext)[2], bool row_vis) {
+        constexpr bool kGeneral = decltype(general_tag)::value;
+        const int n0 = seq(it, it) * kTileN;
+        const bool more1 = it + 1 < ntiles, more2 = it + 2 < ntiles;
+        if (more1) store_k((it + 1) & 1);
+        store_v(it & 1);
+        __syncthreads();
+        if (more2) load_k(seq(it + 2, it));
+        if (more1) {
+            load_v(seq(it + 1, it));
+            scores(snext, (it + 1) & 1);
         }
 
         if constexpr (kGeneral) {  // 64-bit visibility word per row
@@ -290,14 +305,14 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const uint32_t bit = 1u << (8 * (i / 4) + (i % 4));
-                sacc[0][i] = (w0 & bit) ? sacc[0][i] : -INFINITY;
-                sacc[1][i] = (w1 & bit) ? sacc[1][i] : -INFINITY;
+                scur[0][i] = (w0 & bit) ? scur[0][i] : -INFINITY;
+                scur[1][i] = (w1 & bit) ? scur[1][i] : -INFINITY;
             }
         }
 
-        float mloc = fmaxf(sacc[0][0], sacc[1][0]);
+        float mloc = fmaxf(scur[0][0], scur[1][0]);
 #pragma unroll
-        for (int i = 1; i < 16; ++i) mloc = fmaxf(mloc, fmaxf(sacc[0][i], sacc[1][i]));
+        for (int i = 1; i < 16; ++i) mloc = fmaxf(mloc, fmaxf(scur[0][i], scur[1][i]));
         if (!row_vis) mloc = -INFINITY;
         mloc = ksa_pair_max(mloc);
         // lazy rescale: move the reference only when the row maximum outgrows it by 2^kTau
@@ -320,38 +335,58 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
             for (int i = 0; i < 16; i += 2) {
-                const float p0 = ksa_exp2(fmaf(sacc[kb][i], c2, -mc));
-                const float p1 = ksa_exp2(fmaf(sacc[kb][i + 1], c2, -mc));
+                const float p0 = ksa_exp2(fmaf(scur[kb][i], c2, -mc));
+                const float p1 = ksa_exp2(fmaf(scur[kb][i + 1], c2, -mc));
                 const uint32_t pk = Ops::pack2(p0, p1);
                 l_run = Ops::sum2(pk, l_run);
                 pf[kb * 2 + i / 8][(i % 8) / 2] = pk;
             }
+        const int vbuf = it & 1;
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
 #pragma unroll
             for (int b = 0; b < DB; ++b) {
-                const u32x4 a = ksa_read_vt_frag<VROW>(Vs[buf], ks, b, lq, lh);
+                const u32x4 a = ksa_read_vt_frag<VROW>(Vs[vbuf], ks, b, lq, lh);
                 oacc[b] = Ops::mfma(a, pf[ks], oacc[b]);
             }
         }
-    };
-
-    if (ntiles > 0) load_tile(__builtin_amdgcn_readlane(seq_cur, 0));
-    auto advance = [&](int it) {  // after tile `it`: roll the index chunk every 64 tiles
-        if ((it & 63) == 63) {
+        if ((it & 63) == 63) {  // roll the index chunk
             seq_cur = seq_nxt;
             seq_nxt = seq_chunk(it + 1 + 64);
         }
     };
+
+    floatx16 s0[2], s1[2];
+    if (ntiles > 0) {  // prologue: scores of tile 0, then K(1) and V(0) into registers
+        load_k(seq(0, 0));
+        store_k(0);
+        __syncthreads();
+        if (ntiles > 1) load_k(seq(1, 0));
+        load_v(seq(0, 0));
+        scores(s0, 0);
+    }
+    auto copy_scores = [&]() {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) s0[kb][i] = s1[kb][i];
+    };
+    const bool lane_is_text = rv.b_text;
     int it = 0;
-    for (; it < n_a; ++it) {
-        tile_body(std::false_type{}, it, it < nquick ? lane_is_text : true);
-        advance(it);
+    for (; it + 2 <= n_a; it += 2) {
+        step(std::false_type{}, it, s0, s1, it < nquick ? lane_is_text : true);
+        step(std::false_type{}, it + 1, s1, s0, it + 1 < nquick ? lane_is_text : true);
     }
-    for (; it < ntiles; ++it) {
-        tile_body(std::true_type{}, it, true);
-        advance(it);
+    if (it < n_a) {
+        step(std::false_type{}, it, s0, s1, it < nquick ? lane_is_text : true);
+        copy_scores();
+        ++it;
     }
+    for (; it + 2 <= ntiles; it += 2) {
+        step(std::true_type{}, it, s0, s1, true);
+        step(std::true_type{}, it + 1, s1, s0, true);
+    }
+    if (it < ntiles) step(std::true_type{}, it, s0, s1, true);
 
     // ---- epilogue ----
     const float l_tot = ksa_pair_sum(l_run);
@@ -385,53 +420,39 @@ bool stride_ok(int64_t s) { return (s % 8) == 0; }
 
 }  // namespace
 
-extern "C" int ksa_prefill_fwd(const void* q, const void* k, const void* v, const void* kprefix,
-                               const void* vprefix, void* out, float* lse, int batch, int Sq,
-                               int Hq, int Hkv, int D, int dtype, const int64_t* q_strides,
-                               const int64_t* k_strides, const int64_t* v_strides,
-                               const int64_t* kprefix_strides, const int64_t* vprefix_strides,
+extern "C" int ksa_prefill_fwd(const void* q, const void* k, const void* v, void* out, float* lse,
+                               int batch, int Sq, int Hq, int Hkv, int D, int dtype,
+                               const int64_t* q_strides, const int64_t* kv_strides,
                                const int64_t* out_strides, int C, int S, int W, int P,
-                               int skip_old, const int32_t* mask_cnt, const int32_t* mask_idx,
-                               const int32_t* full_cnt, const int32_t* full_idx, int idx_stride,
-                               float scale, void* stream) {
+                               int skip_old, int phys_prefix, const int32_t* mask_cnt,
+                               const int32_t* mask_idx, const int32_t* full_cnt,
+                               const int32_t* full_idx, int idx_stride, float scale, void* stream) {
     if (!q || !k || !v || !out || !mask_cnt || !mask_idx || !full_cnt || !full_idx) return KSA_ERR_NULL;
-    if (!q_strides || !k_strides || !v_strides || !out_strides) return KSA_ERR_NULL;
-    if ((kprefix == nullptr) != (vprefix == nullptr)) return KSA_ERR_NULL;
-    if (kprefix && (!kprefix_strides || !vprefix_strides)) return KSA_ERR_NULL;
+    if (!q_strides || !kv_strides || !out_strides) return KSA_ERR_NULL;
     if (batch <= 0 || Sq <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0) return KSA_ERR_INVALID;
     if (C <= 0 || S <= 0 || W < 0 || P < 0) return KSA_ERR_INVALID;
     if ((int64_t)Sq + P >= (1ll << 30)) return KSA_ERR_INVALID;
-    // K/V rows are addressed with 32-bit byte offsets inside one (batch, head) slice
-    if ((int64_t)Sq * k_strides[1] * 2 >= (1ll << 32) || (int64_t)Sq * v_strides[1] * 2 >= (1ll << 32))
-        return KSA_ERR_INVALID;
-    if (kprefix && ((int64_t)P * kprefix_strides[1] * 2 >= (1ll << 32) ||
-                    (int64_t)P * vprefix_strides[1] * 2 >= (1ll << 32)))
-        return KSA_ERR_INVALID;
     if (dtype != KSA_DTYPE_BF16 && dtype != KSA_DTYPE_F16) return KSA_ERR_UNSUPPORTED;
     const int Sk = Sq + P;
     const int N = (Sk + kTileN - 1) / kTileN;
     if (idx_stride < N) return KSA_ERR_INVALID;
-    if (!kprefix && P > 0) {
+    // K/V rows are addressed with 32-bit byte offsets inside one (batch, head) slice
+    const int64_t kv_rows = phys_prefix ? Sk : Sq;
+    if (kv_rows * kv_strides[1] * 2 >= (1ll << 32)) return KSA_ERR_INVALID;
+    if (!phys_prefix && P > 0) {
         // in-place prefix: row j is in-line row (j/S)*B + C + j%S, which must exist
         const int64_t last = (int64_t)((P - 1) / S) * (C + S) + C + (P - 1) % S;
         if (last >= Sq) return KSA_ERR_INVALID;
     }
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out)) return KSA_ERR_ALIGN;
-    if (kprefix && (!aligned16(kprefix) || !aligned16(vprefix))) return KSA_ERR_ALIGN;
-    for (int i = 0; i < 3; ++i) {
-        if (!stride_ok(q_strides[i]) || !stride_ok(k_strides[i]) || !stride_ok(v_strides[i]) ||
-            !stride_ok(out_strides[i]))
+    for (int i = 0; i < 3; ++i)
+        if (!stride_ok(q_strides[i]) || !stride_ok(kv_strides[i]) || !stride_ok(out_strides[i]))
             return KSA_ERR_ALIGN;
-        if (kprefix && (!stride_ok(kprefix_strides[i]) || !stride_ok(vprefix_strides[i])))
-            return KSA_ERR_ALIGN;
-    }
 
     PrefillParams p{};
     p.q = (const uint16_t*)q;
     p.k = (const uint16_t*)k;
     p.v = (const uint16_t*)v;
-    p.kprefix = (const uint16_t*)kprefix;
-    p.vprefix = (const uint16_t*)vprefix;
     p.out = (uint16_t*)out;
     p.lse = lse;
     p.mask_cnt = mask_cnt;
@@ -443,13 +464,9 @@ extern "C" int ksa_prefill_fwd(const void* q, const void* k, const void* v, cons
     p.Hq = Hq;
     p.Hkv = Hkv;
     p.g = Hq / Hkv;
+    p.phys_prefix = phys_prefix ? 1 : 0;
     p.q_bs = q_strides[0], p.q_rs = q_strides[1], p.q_hs = q_strides[2];
-    p.k_bs = k_strides[0], p.k_rs = k_strides[1], p.k_hs = k_strides[2];
-    p.v_bs = v_strides[0], p.v_rs = v_strides[1], p.v_hs = v_strides[2];
-    if (kprefix) {
-        p.kp_bs = kprefix_strides[0], p.kp_rs = kprefix_strides[1], p.kp_hs = kprefix_strides[2];
-        p.vp_bs = vprefix_strides[0], p.vp_rs = vprefix_strides[1], p.vp_hs = vprefix_strides[2];
-    }
+    p.kv_bs = kv_strides[0], p.kv_rs = kv_strides[1], p.kv_hs = kv_strides[2];
     p.o_bs = out_strides[0], p.o_rs = out_strides[1], p.o_hs = out_strides[2];
     p.lse_bs = (int64_t)Hq * Sq;
     p.lse_hs = Sq;

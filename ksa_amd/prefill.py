@@ -123,27 +123,21 @@ def _lastdim_contig(t):
 
 @torch.library.custom_op("ksa_amd::summary_attn_fwd", mutates_args=())
 def _summary_attn_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
-                      kprefix: Optional[torch.Tensor], vprefix: Optional[torch.Tensor],
                       mask_cnt: torch.Tensor, mask_idx: torch.Tensor, full_cnt: torch.Tensor,
                       full_idx: torch.Tensor, C: int, S: int, W: int, P: int, skip_old: bool,
-                      scale: float, want_lse: bool) -> Tuple[torch.Tensor, torch.Tensor]:
+                      phys_prefix: bool, scale: float, want_lse: bool) -> Tuple[torch.Tensor, torch.Tensor]:
     b, Sq, Hq, D = q.shape
     Hkv = k.shape[2]
     out = torch.empty_like(q)
     lse = torch.empty((b, Hq, Sq) if want_lse else (0,), dtype=torch.float32, device=q.device)
     dims = (0, 1, 2)
-    null3 = ctypes.cast(None, ctypes.POINTER(ctypes.c_int64))
     with torch.cuda.device(q.device):
         rc = _lib.lib().ksa_prefill_fwd(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(),
-            kprefix.data_ptr() if kprefix is not None else None,
-            vprefix.data_ptr() if vprefix is not None else None,
-            out.data_ptr(), lse.data_ptr() if want_lse else None,
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+            lse.data_ptr() if want_lse else None,
             b, Sq, Hq, Hkv, D, _DTYPES[q.dtype],
-            _lib.strides3(q, dims), _lib.strides3(k, dims), _lib.strides3(v, dims),
-            _lib.strides3(kprefix, dims) if kprefix is not None else null3,
-            _lib.strides3(vprefix, dims) if vprefix is not None else null3,
-            _lib.strides3(out, dims), C, S, W, P, int(skip_old),
+            _lib.strides3(q, dims), _lib.strides3(k, dims), _lib.strides3(out, dims),
+            C, S, W, P, int(skip_old), int(phys_prefix),
             mask_cnt.data_ptr(), mask_idx.data_ptr(), full_cnt.data_ptr(), full_idx.data_ptr(),
             mask_idx.shape[-1], float(scale), _lib.stream_ptr(q.device))
     _lib.check(rc, "ksa_prefill_fwd")
@@ -151,10 +145,27 @@ def _summary_attn_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
 
 
 @_summary_attn_fwd.register_fake
-def _(q, k, v, kprefix, vprefix, mask_cnt, mask_idx, full_cnt, full_idx, C, S, W, P, skip_old,
-      scale, want_lse):
+def _(q, k, v, mask_cnt, mask_idx, full_cnt, full_idx, C, S, W, P, skip_old, phys_prefix, scale,
+      want_lse):
     b, Sq, Hq, _ = q.shape
     return torch.empty_like(q), q.new_empty((b, Hq, Sq) if want_lse else (0,), dtype=torch.float32)
+
+
+def _gathered_prefix(t: torch.Tensor, rows: torch.Tensor, P: int) -> torch.Tensor:
+    """[prefix rows | in-line rows] of t [b, Sq, H, D], built with the HIP row mover (the
+    layout the reference makes with torch.cat((t[:, summary_pos], t), dim=1))."""
+    b, Sq, H, D = t.shape
+    full = torch.empty((b, P + Sq, H, D), dtype=t.dtype, device=t.device)
+    lib = _lib.lib()
+    with torch.cuda.device(t.device):
+        st = _lib.stream_ptr(t.device)
+        rc = lib.ksa_copy_rows(t.data_ptr(), full.data_ptr(), rows.data_ptr(), None, 0, 0, P, b, H, D,
+                               _lib.strides3(t, (0, 2, 1)), _lib.strides3(full, (0, 2, 1)), st)
+        _lib.check(rc, "ksa_copy_rows")
+        rc = lib.ksa_copy_rows(t.data_ptr(), full.data_ptr(), None, None, 0, P, Sq, b, H, D,
+                               _lib.strides3(t, (0, 2, 1)), _lib.strides3(full, (0, 2, 1)), st)
+        _lib.check(rc, "ksa_copy_rows")
+    return full
 
 
 def summary_attn_func(q, k, v, chunk_size, summary_num, sliding_chunk_num,
@@ -164,8 +175,10 @@ def summary_attn_func(q, k, v, chunk_size, summary_num, sliding_chunk_num,
     """q [b, Sq, Hq, D]; k, v [b, Sq (+P), Hkv, D]; returns (out [b, Sq, Hq, D], lse or None).
 
     With `summary_pos` (bool [Sq]) the summary rows of k/v form the key prefix, as
-    `torch.cat((k[:, summary_pos], k), dim=1)` does in the reference, but nothing is
-    concatenated: the kernel reads them where they are.  Without it, the first
+    `torch.cat((k[:, summary_pos], k), dim=1)` does in the reference.  For the periodic
+    summary layout (every C text rows followed by S summary rows) nothing is copied: the
+    kernel reads the prefix rows where they are.  Any other `summary_pos` is gathered into
+    a [prefix | in-line] buffer first.  Without `summary_pos`, the first
     `k.shape[1] - q.shape[1]` rows of k/v are taken as an already-built prefix.
     Forward only: tensors that require grad under an enabled grad mode are rejected.
     `return_lse` / `softmax_scale` are extensions (the reference returns lse only for
@@ -174,34 +187,27 @@ def summary_attn_func(q, k, v, chunk_size, summary_num, sliding_chunk_num,
     _check_inputs(q, k, v)
     if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad):
         raise NotImplementedError("ksa_amd implements the prefill forward only; call it under torch.no_grad()")
-    lib = _lib.lib()
     b, Sq, Hq, D = q.shape
     C, S, W = int(chunk_size), int(summary_num), int(sliding_chunk_num)
     assert C > 0 and S > 0 and W >= 0, "chunk_size/summary_num must be positive, sliding_chunk_num >= 0"
     q, k, v = _lastdim_contig(q), _lastdim_contig(k), _lastdim_contig(v)
-    kprefix = vprefix = None
+    phys = False
     if summary_pos is not None:
         assert k.shape[1] == Sq, "with summary_pos, k/v must have the same length as q"
         P, periodic, rows = _analyse_summary_pos(summary_pos, Sq, C, S)
         if P > 0 and not periodic:
-            # arbitrary summary positions: gather just the P prefix rows (not the whole K/V)
-            kprefix = torch.empty((b, P, k.shape[2], D), dtype=k.dtype, device=k.device)
-            vprefix = torch.empty_like(kprefix)
-            with torch.cuda.device(q.device):
-                for src, dst in ((k, kprefix), (v, vprefix)):
-                    rc = lib.ksa_copy_rows(src.data_ptr(), dst.data_ptr(), rows.data_ptr(), None, 0, 0,
-                                           P, b, k.shape[2], D, _lib.strides3(src, (0, 2, 1)),
-                                           _lib.strides3(dst, (0, 2, 1)), _lib.stream_ptr(q.device))
-                    _lib.check(rc, "ksa_copy_rows")
+            k, v = _gathered_prefix(k, rows, P), _gathered_prefix(v, rows, P)
+            phys = True
     else:
         P = k.shape[1] - Sq
         assert P >= 0, "k/v must be at least as long as q"
-        if P > 0:
-            kprefix, vprefix = k[:, :P], v[:, :P]
-            k, v = k[:, P:], v[:, P:]
+        phys = P > 0
+    if k.stride() != v.stride():
+        v = v.contiguous()
+        k = k.contiguous()
     idx = _cached_index(Sq, C, S, W, P, skip_old_summary, q.device)
     scale = float(D) ** -0.5 if softmax_scale is None else float(softmax_scale)
     out, lse = torch.ops.ksa_amd.summary_attn_fwd(
-        q, k, v, kprefix, vprefix, idx[0], idx[1], idx[2], idx[3], C, S, W, P,
-        bool(skip_old_summary), scale, bool(return_lse))
+        q, k, v, idx[0], idx[1], idx[2], idx[3], C, S, W, P,
+        bool(skip_old_summary), phys, scale, bool(return_lse))
     return out, (lse if return_lse else None)
