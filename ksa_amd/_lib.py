@@ -8,7 +8,8 @@ import os
 import torch  # noqa: F401  (must be imported first so that its HIP runtime is the one in the process)
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libksa_hip.so")
+# KSA_AMD_LIB selects another build of the same library (e.g. a profiling variant)
+LIB_PATH = os.environ.get("KSA_AMD_LIB") or os.path.join(_HERE, "libksa_hip.so")
 _lib = None
 
 _i32p = ctypes.POINTER(ctypes.c_int32)

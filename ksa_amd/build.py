@@ -13,12 +13,15 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    # scores never hold NaN unless the inputs do; without this every fmax is preceded by a
+    # canonicalising v_max
+    "-fno-honor-nans",
 ]
 
 
-def build(verbose: bool = False, extra_flags=()) -> str:
+def build(verbose: bool = False, extra_flags=(), out: str = LIB) -> str:
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc, *FLAGS, *extra_flags, "-I", CSRC, "-o", LIB] + [os.path.join(CSRC, s) for s in SOURCES]
+    cmd = [hipcc, *FLAGS, *extra_flags, "-I", CSRC, "-o", out] + [os.path.join(CSRC, s) for s in SOURCES]
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)
@@ -28,7 +31,7 @@ def build(verbose: bool = False, extra_flags=()) -> str:
         raise RuntimeError(f"hipcc failed ({res.returncode}):\n{err}")
     if verbose and err.strip():
         print(err, file=sys.stderr)
-    return LIB
+    return out
 
 
 if __name__ == "__main__":

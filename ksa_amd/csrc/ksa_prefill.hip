@@ -94,7 +94,10 @@ __device__ __forceinline__ RowVis ksa_row_vis(const KsaMask& mk, int q) {
     return r;
 }
 
-template <typename T, int D>
+// kRegular: every listed key tile lies entirely in the summary prefix or entirely in the
+// in-line region and inside the key axis (P and Sk multiples of 64), and in-place prefix
+// rows of one thread differ by a uniform step; then tile addressing is branch-free.
+template <typename T, int D, bool kRegular>
 __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillParams p) {
     using Ops = KsaOps<T>;
     constexpr int KS = D / 16;       // contraction steps of K Q^T
@@ -164,6 +167,15 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
 
     // tile -> (uniform byte offset, uniform per-load step, per-thread byte offsets)
     auto tile_src = [&](int n0, uint32_t& ubase, uint32_t& ustep, uint32_t (&voff)[KLD]) {
+        if constexpr (kRegular) {
+            const bool in_main = phys || n0 >= mk.P;
+            ubase = in_main ? (uint32_t)(phys ? n0 : n0 - mk.P) * rb : (uint32_t)(n0 / mk.S) * Bblk * rb;
+            ustep = in_main ? step_main : step_pre;
+            const uint32_t t = in_main ? thr_main : thr_pre;
+#pragma unroll
+            for (int i = 0; i < KLD; ++i) voff[i] = t;
+            return;
+        }
         const bool in_main = (phys || n0 >= mk.P) && n0 + kTileN <= mk.Sk;
         if (in_main) {
             ubase = (uint32_t)(phys ? n0 : n0 - mk.P) * rb;
@@ -255,7 +267,9 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
     for (int b = 0; b < DB; ++b)
 #pragma unroll
         for (int i = 0; i < 16; ++i) oacc[b][i] = 0.f;
-    float m_ref = -INFINITY;  // reference maximum of the exponents (raw score units)
+    // reference maximum of the exponents (raw score units); a finite "minus huge" start
+    // value makes the first visible tile rescale the (still zero) accumulators by 0
+    float m_ref = -1e30f;
     float l_run = 0.f;        // this lane's half of the row sum
     const float c2 = p.scale_log2;
 
@@ -280,15 +294,14 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
     auto step = [&](auto general_tag, int it, floatx16 (&scur)[2], floatx16 (&snext)[2], bool row_vis) {
         constexpr bool kGeneral = decltype(general_tag)::value;
         const int n0 = seq(it, it) * kTileN;
-        const bool more1 = it + 1 < ntiles, more2 = it + 2 < ntiles;
-        if (more1) store_k((it + 1) & 1);
+        // Past the end of the walk the pipeline keeps running on the last tile (loads) and
+        // on stale LDS contents (scores); those results are never used.
+        store_k((it + 1) & 1);
         store_v(it & 1);
         __syncthreads();
-        if (more2) load_k(seq(it + 2, it));
-        if (more1) {
-            load_v(seq(it + 1, it));
-            scores(snext, (it + 1) & 1);
-        }
+        load_k(seq(min(it + 2, ntiles - 1), it));
+        load_v(seq(min(it + 1, ntiles - 1), it));
+        scores(snext, (it + 1) & 1);
 
         if constexpr (kGeneral) {  // 64-bit visibility word per row
             const int kv = n0 + lane;
@@ -316,19 +329,18 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
         if (!row_vis) mloc = -INFINITY;
         mloc = ksa_pair_max(mloc);
         // lazy rescale: move the reference only when the row maximum outgrows it by 2^kTau
-        const bool bump = (mloc - m_ref) * c2 > kTau || m_ref == -INFINITY;
-        const float m_new = bump ? mloc : m_ref;
-        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-        if (__any(bump && mloc != -INFINITY)) {
-            const float alpha = ksa_exp2((m_ref - m_safe) * c2);
+        const bool bump = (mloc - m_ref) * c2 > kTau;
+        if (__any(bump)) {
+            const float m_new = bump ? mloc : m_ref;
+            const float alpha = ksa_exp2((m_ref - m_new) * c2);
+            m_ref = m_new;
             l_run *= alpha;
 #pragma unroll
             for (int b = 0; b < DB; ++b)
 #pragma unroll
                 for (int i = 0; i < 16; ++i) oacc[b][i] *= alpha;
         }
-        m_ref = m_new;
-        const float mc = row_vis ? m_safe * c2 : INFINITY;
+        const float mc = row_vis ? m_ref * c2 : INFINITY;
 
         u32x4 pf[4];
 #pragma unroll
@@ -361,7 +373,7 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
         load_k(seq(0, 0));
         store_k(0);
         __syncthreads();
-        if (ntiles > 1) load_k(seq(1, 0));
+        load_k(seq(min(1, ntiles - 1), 0));
         load_v(seq(0, 0));
         scores(s0, 0);
     }
@@ -411,7 +423,14 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
 template <typename T, int D>
 int launch(const PrefillParams& p, int batch, hipStream_t stream) {
     dim3 grid(p.M * p.Hq, batch);
-    hipLaunchKernelGGL((ksa_prefill_kernel<T, D>), grid, dim3(kThreads), 0, stream, p);
+    constexpr int RSTEP = kThreads / (D / 8);
+    const KsaMask& mk = p.mk;
+    const bool prefix_ok = mk.P == 0 || p.phys_prefix || (RSTEP % mk.S == 0 && mk.P % kTileN == 0);
+    const bool regular = prefix_ok && mk.Sk % kTileN == 0;
+    if (regular)
+        hipLaunchKernelGGL((ksa_prefill_kernel<T, D, true>), grid, dim3(kThreads), 0, stream, p);
+    else
+        hipLaunchKernelGGL((ksa_prefill_kernel<T, D, false>), grid, dim3(kThreads), 0, stream, p);
     return ksa_check_launch();
 }
 
