@@ -103,7 +103,7 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
     constexpr int KS = D / 16;       // contraction steps of K Q^T
     constexpr int DB = D / 32;       // 32-row blocks of O^T
     constexpr int KROW = D + 8;      // padded LDS row of K (elements)
-    constexpr int VROW = D + 16;     // padded LDS row of V (stride = 8 banks mod 64)
+    constexpr int VROW = D + 32;     // padded LDS row of V (stride = 16 banks mod 64)
     constexpr int CPR = D / 8;       // 16-byte chunks per K/V row
     constexpr int KLD = (kTileN * CPR) / kThreads;  // K (and V) loads per thread
     constexpr int RSTEP = kThreads / CPR;           // row distance between a thread's loads
@@ -167,14 +167,8 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
 
     // tile -> (uniform byte offset, uniform per-load step, per-thread byte offsets)
     auto tile_src = [&](int n0, uint32_t& ubase, uint32_t& ustep, uint32_t (&voff)[KLD]) {
-        if constexpr (kRegular) {
-            const bool in_main = phys || n0 >= mk.P;
-            ubase = in_main ? (uint32_t)(phys ? n0 : n0 - mk.P) * rb : (uint32_t)(n0 / mk.S) * Bblk * rb;
-            ustep = in_main ? step_main : step_pre;
-            const uint32_t t = in_main ? thr_main : thr_pre;
-#pragma unroll
-            for (int i = 0; i < KLD; ++i) voff[i] = t;
-            return;
+        if constexpr (kRegular) {  // not used: regular tiles take the precomputed offset word
+            (void)n0;
         }
         const bool in_main = (phys || n0 >= mk.P) && n0 + kTileN <= mk.Sk;
         if (in_main) {
@@ -195,21 +189,31 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
         }
     };
 
+    // Regular tiles: uniform offset word = byte offset of the tile's first row | 1 if the
+    // tile lies in the in-line region (computed per lane when the walk order is fetched).
+    auto tile_word = [&](int n) -> uint32_t {
+        const int n0 = n * kTileN;
+        const bool in_main = phys || n0 >= mk.P;
+        return in_main ? ((uint32_t)(phys ? n0 : n0 - mk.P) * rb) | 1u
+                       : (uint32_t)(n0 / mk.S) * Bblk * rb;
+    };
     u32x4 kreg[KLD];
     u32x4 vreg[KLD];
-    auto load_k = [&](int n) {
+    auto load_kv = [&](const char* base, u32x4 (&reg)[KLD], int n, uint32_t word) {
         uint32_t ub, us, vo[KLD];
-        tile_src(n * kTileN, ub, us, vo);
+        if constexpr (kRegular) {
+            const bool in_main = word & 1u;
+            ub = word & ~1u;
+            us = in_main ? step_main : step_pre;
+            const uint32_t t = in_main ? thr_main : thr_pre;
+#pragma unroll
+            for (int i = 0; i < KLD; ++i) vo[i] = t;
+        } else {
+            tile_src(n * kTileN, ub, us, vo);
+        }
 #pragma unroll
         for (int i = 0; i < KLD; ++i)
-            kreg[i] = *reinterpret_cast<const u32x4*>(kbase + (ub + us * i) + vo[i]);
-    };
-    auto load_v = [&](int n) {
-        uint32_t ub, us, vo[KLD];
-        tile_src(n * kTileN, ub, us, vo);
-#pragma unroll
-        for (int i = 0; i < KLD; ++i)
-            vreg[i] = *reinterpret_cast<const u32x4*>(vbase + (ub + us * i) + vo[i]);
+            reg[i] = *reinterpret_cast<const u32x4*>(base + (ub + us * i) + vo[i]);
     };
     auto store_k = [&](int buf) {
 #pragma unroll
@@ -256,10 +260,16 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
     auto seq_chunk = [&](int base) { return base + lane < ntiles ? tile_at(base + lane) : 0; };
     int seq_cur = seq_chunk(0);
     int seq_nxt = seq_chunk(64);
-    auto seq = [&](int i, int it) {  // entry i in {it, it+1, it+2} while processing tile it
-        const int c = (i >> 6) - (it >> 6);
-        return c == 0 ? __builtin_amdgcn_readlane(seq_cur, i & 63)
-                      : __builtin_amdgcn_readlane(seq_nxt, i & 63);
+    uint32_t word_cur = kRegular ? tile_word(seq_cur) : 0u;
+    uint32_t word_nxt = kRegular ? tile_word(seq_nxt) : 0u;
+    // entry i in {it, it+1, it+2} while processing tile it
+    auto seq = [&](int i, int it) {
+        const int src = (i >> 6) == (it >> 6) ? seq_cur : seq_nxt;
+        return __builtin_amdgcn_readlane(src, i & 63);
+    };
+    auto seq_word = [&](int i, int it) {
+        const uint32_t src = (i >> 6) == (it >> 6) ? word_cur : word_nxt;
+        return (uint32_t)__builtin_amdgcn_readlane((int)src, i & 63);
     };
 
     floatx16 oacc[DB];
@@ -296,11 +306,14 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
         const int n0 = seq(it, it) * kTileN;
         // Past the end of the walk the pipeline keeps running on the last tile (loads) and
         // on stale LDS contents (scores); those results are never used.
+        const int ik = min(it + 2, ntiles - 1), iv = min(it + 1, ntiles - 1);
+        const int nk = seq(ik, it), nv = seq(iv, it);
+        const uint32_t wk = seq_word(ik, it), wv = seq_word(iv, it);
         store_k((it + 1) & 1);
         store_v(it & 1);
         __syncthreads();
-        load_k(seq(min(it + 2, ntiles - 1), it));
-        load_v(seq(min(it + 1, ntiles - 1), it));
+        load_kv(kbase, kreg, nk, wk);
+        load_kv(vbase, vreg, nv, wv);
         scores(snext, (it + 1) & 1);
 
         if constexpr (kGeneral) {  // 64-bit visibility word per row
@@ -364,17 +377,20 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
         }
         if ((it & 63) == 63) {  // roll the index chunk
             seq_cur = seq_nxt;
+            word_cur = word_nxt;
             seq_nxt = seq_chunk(it + 1 + 64);
+            word_nxt = kRegular ? tile_word(seq_nxt) : 0u;
         }
     };
 
     floatx16 s0[2], s1[2];
     if (ntiles > 0) {  // prologue: scores of tile 0, then K(1) and V(0) into registers
-        load_k(seq(0, 0));
+        load_kv(kbase, kreg, seq(0, 0), seq_word(0, 0));
         store_k(0);
         __syncthreads();
-        load_k(seq(min(1, ntiles - 1), 0));
-        load_v(seq(0, 0));
+        const int i1 = min(1, ntiles - 1);
+        load_kv(kbase, kreg, seq(i1, 0), seq_word(i1, 0));
+        load_kv(vbase, vreg, seq(0, 0), seq_word(0, 0));
         scores(s0, 0);
     }
     auto copy_scores = [&]() {
