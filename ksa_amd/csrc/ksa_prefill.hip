@@ -314,7 +314,7 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
         __syncthreads();
         load_kv(kbase, kreg, nk, wk);
         load_kv(vbase, vreg, nv, wv);
-        scores(snext, (it + 1) & 1);
+        if constexpr (kGeneral) scores(snext, (it + 1) & 1);
 
         if constexpr (kGeneral) {  // 64-bit visibility word per row
             const int kv = n0 + lane;
@@ -336,43 +336,115 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
             }
         }
 
-        float mloc = fmaxf(scur[0][0], scur[1][0]);
-#pragma unroll
-        for (int i = 1; i < 16; ++i) mloc = fmaxf(mloc, fmaxf(scur[0][i], scur[1][i]));
-        if (!row_vis) mloc = -INFINITY;
-        mloc = ksa_pair_max(mloc);
-        // lazy rescale: move the reference only when the row maximum outgrows it by 2^kTau
-        const bool bump = (mloc - m_ref) * c2 > kTau;
-        if (__any(bump)) {
-            const float m_new = bump ? mloc : m_ref;
-            const float alpha = ksa_exp2((m_ref - m_new) * c2);
-            m_ref = m_new;
-            l_run *= alpha;
-#pragma unroll
-            for (int b = 0; b < DB; ++b)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) oacc[b][i] *= alpha;
-        }
-        const float mc = row_vis ? m_ref * c2 : INFINITY;
-
+        // Probabilities relative to the current reference.  The row maximum is computed
+        // only where it is needed: always on the masked tiles of phase B; on phase A tiles
+        // only after the fact, when a row has no reference yet or its tile sum shows that the
+        // exponents outgrew the reference (then the tile's probabilities are redone).
+        float l_tile = 0.f;
         u32x4 pf[4];
+        float mc = row_vis ? m_ref * c2 : INFINITY;
+        // four probabilities (two packed pairs) of 16-key group g, half h
+        auto prob4 = [&](int g, int h) {
+            const int kb = g >> 1, i0 = 8 * (g & 1) + 4 * h;
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int i = 0; i < 16; i += 2) {
-                const float p0 = ksa_exp2(fmaf(scur[kb][i], c2, -mc));
-                const float p1 = ksa_exp2(fmaf(scur[kb][i + 1], c2, -mc));
+            for (int j = 0; j < 2; ++j) {
+                const float p0 = ksa_exp2(fmaf(scur[kb][i0 + 2 * j], c2, -mc));
+                const float p1 = ksa_exp2(fmaf(scur[kb][i0 + 2 * j + 1], c2, -mc));
                 const uint32_t pk = Ops::pack2(p0, p1);
-                l_run = Ops::sum2(pk, l_run);
-                pf[kb * 2 + i / 8][(i % 8) / 2] = pk;
+                l_tile = Ops::sum2(pk, l_tile);
+                pf[g][2 * h + j] = pk;
             }
-        const int vbuf = it & 1;
+        };
+        auto probabilities = [&]() {
+            mc = row_vis ? m_ref * c2 : INFINITY;
+            l_tile = 0.f;
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
+            for (int g = 0; g < 4; ++g) {
+                prob4(g, 0);
+                prob4(g, 1);
+            }
+        };
+        // move the reference of the rows whose maximum outgrew it (or that have none yet)
+        auto rebase = [&]() {
+            float mloc = fmaxf(scur[0][0], scur[1][0]);
 #pragma unroll
-            for (int b = 0; b < DB; ++b) {
-                const u32x4 a = ksa_read_vt_frag<VROW>(Vs[vbuf], ks, b, lq, lh);
-                oacc[b] = Ops::mfma(a, pf[ks], oacc[b]);
+            for (int i = 1; i < 16; ++i) mloc = fmaxf(mloc, fmaxf(scur[0][i], scur[1][i]));
+            if (!row_vis) mloc = -INFINITY;
+            mloc = ksa_pair_max(mloc);
+            const bool bump = (mloc - m_ref) * c2 > kTau;
+            if (__any(bump)) {
+                const float m_new = bump ? mloc : m_ref;
+                const float alpha = ksa_exp2((m_ref - m_new) * c2);
+                m_ref = m_new;
+                l_run *= alpha;
+#pragma unroll
+                for (int b = 0; b < DB; ++b)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) oacc[b][i] *= alpha;
+            }
+        };
+        if constexpr (kGeneral) {
+            rebase();
+            probabilities();
+        } else {
+            // Four stages: the score MFMAs of contraction steps [g*SPS, (g+1)*SPS) of the NEXT
+            // tile interleaved with the probabilities of key group g of THIS tile.  The fences
+            // pin this order: operand reads, half of the vector work (covers the LDS latency),
+            // then the MFMAs with the other half in their shadow.
+            constexpr int SPS = KS / 4;
+            const int kbuf = (it + 1) & 1;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                u32x4 kf[SPS][2];
+#pragma unroll
+                for (int t = 0; t < SPS; ++t)
+#pragma unroll
+                    for (int kb = 0; kb < 2; ++kb)
+                        kf[t][kb] = *reinterpret_cast<const u32x4*>(
+                            &Ks[kbuf][(kb * 32 + lq) * KROW + 16 * (g * SPS + t) + 8 * lh]);
+                __builtin_amdgcn_sched_barrier(0);
+                prob4(g, 0);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int t = 0; t < SPS; ++t)
+#pragma unroll
+                    for (int kb = 0; kb < 2; ++kb) {
+                        if (g == 0 && t == 0) {
+                            floatx16 z;
+#pragma unroll
+                            for (int i = 0; i < 16; ++i) z[i] = 0.f;
+                            snext[kb] = Ops::mfma(kf[t][kb], qf[0], z);
+                        } else {
+                            snext[kb] = Ops::mfma(kf[t][kb], qf[g * SPS + t], snext[kb]);
+                        }
+                    }
+                prob4(g, 1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            // 2^24: some exponent exceeded the reference by more than ~19; also true for the
+            // first visible tile of a row (reference still "minus huge" -> infinite sum)
+            if (__any(l_tile > 16777216.f)) {
+                rebase();
+                probabilities();
+            }
+        }
+        l_run += l_tile;
+
+        // O^T += V^T P^T, V operands read one 16-key step ahead of their MFMAs
+        {
+            u32x4 vf[2][DB];
+#pragma unroll
+            for (int b = 0; b < DB; ++b) vf[0][b] = ksa_read_vt_frag<VROW>(Vs[it & 1], 0, b, lq, lh);
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+                if (ks < 3) {
+#pragma unroll
+                    for (int b = 0; b < DB; ++b)
+                        vf[(ks + 1) & 1][b] = ksa_read_vt_frag<VROW>(Vs[it & 1], ks + 1, b, lq, lh);
+                }
+#pragma unroll
+                for (int b = 0; b < DB; ++b) oacc[b] = Ops::mfma(vf[ks & 1][b], pf[ks], oacc[b]);
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
         if ((it & 63) == 63) {  // roll the index chunk
