@@ -243,3 +243,40 @@ def test_prefill_rejects_bad_inputs():
     qg = q.clone().requires_grad_(True)
     with pytest.raises(NotImplementedError):
         ksa_amd.summary_attn_func(qg, q, q, 128, 8, 1)
+
+
+def test_prefill_growing_scores_rebase():
+    """Scores that grow strongly along the key axis (later tiles exceed every earlier row
+    maximum by far) force the soft-max reference to move many times, including on tiles that
+    take the no-maximum fast path; a stale reference would overflow or lose the early keys."""
+    Sq, Hq, Hkv, D, C, S, W = 64 * 136, 4, 2, 128, 128, 8, 2
+    q, k, v = make_qkv(Sq, Hq, Hkv, D, seed=5, scaled=False)
+    # key norm grows with position: summary rows (the prefix tiles) of later chunks get much
+    # larger logits than those of earlier chunks
+    ramp = torch.linspace(0.2, 6.0, Sq)[:, None, None]
+    k = (k.float() * ramp).to(torch.bfloat16)
+    q = (q.float() * 2.0).to(torch.bfloat16)
+    sp = O.summary_positions(Sq, C, S)
+    got, lse = _run_prefill(q, k, v, C, S, W, sp)
+    rows = np.r_[0:300, Sq - 600:Sq].astype(np.int32)
+    want, wlse = c_oracle.attention_rows(to_np(q), to_np(k), to_np(v), C, S, W, summary_pos=sp, rows=rows)
+    assert np.isfinite(got).all()
+    err = np.abs(got[rows] - want).max()
+    assert err <= ATOL * max(1.0, np.abs(want).max()), err
+    assert np.abs(lse[:, rows] - wlse).max() <= 0.1
+
+
+def test_prefill_decreasing_scores():
+    """The opposite order: the first tiles hold the largest logits, everything later is far
+    below the reference (probabilities underflow gracefully, nothing is rescaled)."""
+    Sq, Hq, Hkv, D, C, S, W = 48 * 136, 4, 2, 128, 128, 8, 3
+    q, k, v = make_qkv(Sq, Hq, Hkv, D, seed=6, scaled=False)
+    ramp = torch.linspace(6.0, 0.2, Sq)[:, None, None]
+    k = (k.float() * ramp).to(torch.bfloat16)
+    q = (q.float() * 2.0).to(torch.bfloat16)
+    sp = O.summary_positions(Sq, C, S)
+    got, _ = _run_prefill(q, k, v, C, S, W, sp)
+    rows = np.r_[0:200, Sq - 400:Sq].astype(np.int32)
+    want, _ = c_oracle.attention_rows(to_np(q), to_np(k), to_np(v), C, S, W, summary_pos=sp, rows=rows)
+    err = np.abs(got[rows] - want).max()
+    assert err <= ATOL * max(1.0, np.abs(want).max()), err
