@@ -131,6 +131,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--skip-decode", action="store_true")
     ap.add_argument("--skip-prefill", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one ksa_copy_rows of 1 GiB (a plain copy kernel of known size, "
+                         "used to scale the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (see DESIGN.md, "
@@ -153,6 +156,16 @@ def main():
         "data": "synthetic (seed 0; q,k,v ~ N(0,1)/sqrt(128) for prefill, N(0,1) for decode)",
         "device": torch.cuda.get_device_name(0), "cu_count": _lib.lib().ksa_device_cu_count(),
     }
+
+    if args.calibrate_copy:
+        from ksa_amd.cache import _move_rows
+        rows = 2 ** 30 // (8 * 128 * 2)          # 1 GiB = rows x 8 heads x 128 dims x 2 B
+        src = torch.ones(1, 8, rows, 128, dtype=torch.bfloat16, device=dev)
+        dst = torch.empty_like(src)
+        _move_rows(src, dst, rows)
+        torch.cuda.synchronize()
+        result["calibration_copy_bytes"] = rows * 8 * 128 * 2
+        del src, dst
 
     # ------------------------------------------------------------------ prefill
     if not args.skip_prefill:
@@ -249,6 +262,18 @@ def main():
         except Exception as e:  # the baseline is a reported extra, never the measured path
             result["cpu_baseline"] = {"error": repr(e)}
 
+    # HBM traffic per launch comes from a separate rocprofv3 --pmc measurement (FETCH_SIZE and
+    # WRITE_SIZE, scaled by a copy kernel of known size); the summary is kept under profiles/
+    tfile = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if os.path.exists(tfile):
+        try:
+            t = json.load(open(tfile))
+            if "roofline" in result and result.get("config", {}).get("workload") == t.get("prefill_workload"):
+                result["roofline"]["traffic"] = t.get("prefill_bytes_per_launch")
+            if "decode" in result and result["decode"]["workload"] == t.get("decode_workload"):
+                result["decode"]["roofline"]["traffic"] = t.get("decode_bytes_per_launch")
+        except Exception:
+            pass
     print(json.dumps(result))
 
 

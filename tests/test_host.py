@@ -45,7 +45,8 @@ def test_error_codes_before_launch():
                             null3, null3, 1.0, 1, None, 0, None) == -2
     assert L.ksa_decode_workspace_bytes(64, 32, 8, 1, 128, 1) == 0
     assert L.ksa_decode_workspace_bytes(64, 32, 8, 1, 128, 2) == 64 * 8 * 2 * 32 * 130 * 4
-    assert L.ksa_decode_auto_splits(64, 8, 17288) == 2
+    assert L.ksa_decode_auto_splits(64, 8, 17288) == 1
+    assert L.ksa_decode_auto_splits(8, 8, 17288) == 8
     assert L.ksa_decode_auto_splits(1, 8, 100) == 1
     assert 1 <= L.ksa_decode_auto_splits(1, 8, 100000) <= 64
 
