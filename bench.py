@@ -66,7 +66,7 @@ def time_region(fn, steps, warmup):
     return t1 - t0, e0.elapsed_time(e1)
 
 
-def cpu_baseline_prefill(chunks, Hq, Hkv, D, C, S, W, tiles_per_mtile, budget_s=12.0):
+def cpu_baseline_prefill(chunks, Hq, Hkv, D, C, S, W, tiles_per_mtile, budget_s=20.0):
     """The reference's CPU path (block mode, restated in oracle/cpu_path.py) on a bounded
     sample of 4096-row query blocks; rate in the same non-empty-block TFLOP/s unit."""
     import torch
@@ -77,7 +77,7 @@ def cpu_baseline_prefill(chunks, Hq, Hkv, D, C, S, W, tiles_per_mtile, budget_s=
     k = (torch.randn(Sq, Hkv, D) * scale).bfloat16().float()
     v = (torch.randn(Sq, Hkv, D) * scale).bfloat16().float()
     nblk = -(-Sq // cpu_path.BLOCK_ROWS)
-    pick = sorted({0, nblk // 2, nblk - 1})
+    pick = sorted({0, nblk // 4, nblk // 2, (3 * nblk) // 4, nblk - 1})
     # non-empty 128 x 64 tiles of the sampled rows come from the (parity-checked) block index
     done_tiles, t_used, blocks = 0, 0.0, []
     for bi in pick:
@@ -102,7 +102,7 @@ def cpu_baseline_prefill(chunks, Hq, Hkv, D, C, S, W, tiles_per_mtile, budget_s=
     }
 
 
-def cpu_baseline_decode(Hq, Hkv, D, rows, nseq=2):
+def cpu_baseline_decode(Hq, Hkv, D, rows, nseq=4):
     import torch
     from oracle import cpu_path
     torch.manual_seed(0)
@@ -111,7 +111,7 @@ def cpu_baseline_decode(Hq, Hkv, D, rows, nseq=2):
     v = torch.randn(nseq, Hkv, rows, D)
     cpu_path.decode_sdpa(q, k, v, Hq // Hkv)
     t0 = time.perf_counter()
-    reps = 3
+    reps = 5
     for _ in range(reps):
         cpu_path.decode_sdpa(q, k, v, Hq // Hkv)
     dt = (time.perf_counter() - t0) / reps
