@@ -300,21 +300,38 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
     };
 
     // One pipeline step for tile `it`: its scores are in `scur`; the scores of tile it+1
-    // are produced into `snext`.  On entry the registers hold K(it+1) and V(it).
+    // are produced into `snext`.  On entry LDS holds (or is being written with) K(it+1) and
+    // V(it), and the registers hold K(it+2) and V(it+1).  The barrier publishes the LDS tiles;
+    // the staging registers are written to the buffers freed by the previous step and refilled
+    // from global memory in the shadow of the second product's MFMAs, so that no wave ever
+    // sits in a block of loads or LDS stores with the matrix unit idle.
     auto step = [&](auto general_tag, int it, floatx16 (&scur)[2], floatx16 (&snext)[2], bool row_vis) {
         constexpr bool kGeneral = decltype(general_tag)::value;
         const int n0 = seq(it, it) * kTileN;
         // Past the end of the walk the pipeline keeps running on the last tile (loads) and
         // on stale LDS contents (scores); those results are never used.
-        const int ik = min(it + 2, ntiles - 1), iv = min(it + 1, ntiles - 1);
+        const int ik = min(it + 3, ntiles - 1), iv = min(it + 2, ntiles - 1);
         const int nk = seq(ik, it), nv = seq(iv, it);
         const uint32_t wk = seq_word(ik, it), wv = seq_word(iv, it);
-        store_k((it + 1) & 1);
-        store_v(it & 1);
         __syncthreads();
-        load_kv(kbase, kreg, nk, wk);
-        load_kv(vbase, vreg, nv, wv);
-        if constexpr (kGeneral) scores(snext, (it + 1) & 1);
+
+        // MFMA operands that come from LDS travel through a rolling queue of kQueue fragments:
+        // the read for operand j + kQueue is issued right behind MFMA j, through the score
+        // product (K fragments), across its end (the first V fragments) and through the second
+        // product, so every read has kQueue MFMAs plus the vector work between them to land.
+        constexpr int kQueue = 4;
+        constexpr int NQK = 2 * KS;   // score MFMAs: contraction step s = j / 2, key block kb = j % 2
+        constexpr int NPV = 4 * DB;   // second-product MFMAs: key step ks = j / DB, dim block j % DB
+        const uint16_t* ksrc = Ks[(it + 1) & 1];
+        const uint16_t* vsrc = Vs[it & 1];
+        auto kfrag = [&](int j) {
+            return *reinterpret_cast<const u32x4*>(&ksrc[((j & 1) * 32 + lq) * KROW + 16 * (j >> 1) + 8 * lh]);
+        };
+        auto vfrag = [&](int j) { return ksa_read_vt_frag<VROW>(vsrc, j / DB, j % DB, lq, lh); };
+        u32x4 fq[kQueue];
+#pragma unroll
+        for (int j = 0; j < kQueue; ++j) fq[j] = kfrag(j);
+        __builtin_amdgcn_sched_barrier(0);
 
         if constexpr (kGeneral) {  // 64-bit visibility word per row
             const int kv = n0 + lane;
@@ -343,26 +360,20 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
         float l_tile = 0.f;
         u32x4 pf[4];
         float mc = row_vis ? m_ref * c2 : INFINITY;
-        // four probabilities (two packed pairs) of 16-key group g, half h
-        auto prob4 = [&](int g, int h) {
-            const int kb = g >> 1, i0 = 8 * (g & 1) + 4 * h;
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                const float p0 = ksa_exp2(fmaf(scur[kb][i0 + 2 * j], c2, -mc));
-                const float p1 = ksa_exp2(fmaf(scur[kb][i0 + 2 * j + 1], c2, -mc));
-                const uint32_t pk = Ops::pack2(p0, p1);
-                l_tile = Ops::sum2(pk, l_tile);
-                pf[g][2 * h + j] = pk;
-            }
+        // probability pair c (0..15): keys of 16-key group c / 4, packed word c % 4
+        auto prob2 = [&](int c) {
+            const int g = c >> 2, kb = g >> 1, i0 = 8 * (g & 1) + 2 * (c & 3);
+            const float p0 = ksa_exp2(fmaf(scur[kb][i0], c2, -mc));
+            const float p1 = ksa_exp2(fmaf(scur[kb][i0 + 1], c2, -mc));
+            const uint32_t pk = Ops::pack2(p0, p1);
+            l_tile = Ops::sum2(pk, l_tile);
+            pf[g][c & 3] = pk;
         };
         auto probabilities = [&]() {
             mc = row_vis ? m_ref * c2 : INFINITY;
             l_tile = 0.f;
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                prob4(g, 0);
-                prob4(g, 1);
-            }
+            for (int c = 0; c < 16; ++c) prob2(c);
         };
         // move the reference of the rows whose maximum outgrew it (or that have none yet)
         auto rebase = [&]() {
@@ -385,67 +396,74 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
         };
         if constexpr (kGeneral) {
             rebase();
-            probabilities();
-        } else {
-            // Four stages: the score MFMAs of contraction steps [g*SPS, (g+1)*SPS) of the NEXT
-            // tile interleaved with the probabilities of key group g of THIS tile.  The fences
-            // pin this order: operand reads, half of the vector work (covers the LDS latency),
-            // then the MFMAs with the other half in their shadow.
-            constexpr int SPS = KS / 4;
-            const int kbuf = (it + 1) & 1;
+            mc = row_vis ? m_ref * c2 : INFINITY;
+        }
+
+        // Score MFMAs of the NEXT tile with the probability pairs of THIS tile between them.
+        // The fences pin the order; kLead pairs run first and cover the first operand reads.
+        constexpr int CPM = 16 / NQK;            // probability pairs per score MFMA
+        constexpr int kLead = 3 * CPM;
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                u32x4 kf[SPS][2];
+        for (int c = 0; c < kLead; ++c) prob2(c);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int t = 0; t < SPS; ++t)
+        for (int j = 0; j < NQK; ++j) {
+            const int kb = j & 1;
+            if (j < 2) {
+                floatx16 z;
 #pragma unroll
-                    for (int kb = 0; kb < 2; ++kb)
-                        kf[t][kb] = *reinterpret_cast<const u32x4*>(
-                            &Ks[kbuf][(kb * 32 + lq) * KROW + 16 * (g * SPS + t) + 8 * lh]);
-                __builtin_amdgcn_sched_barrier(0);
-                prob4(g, 0);
-                __builtin_amdgcn_sched_barrier(0);
+                for (int i = 0; i < 16; ++i) z[i] = 0.f;
+                snext[kb] = Ops::mfma(fq[j % kQueue], qf[0], z);
+            } else {
+                snext[kb] = Ops::mfma(fq[j % kQueue], qf[j >> 1], snext[kb]);
+            }
+            fq[j % kQueue] = (j + kQueue < NQK) ? kfrag(j + kQueue) : vfrag(j + kQueue - NQK);
 #pragma unroll
-                for (int t = 0; t < SPS; ++t)
+            for (int c = kLead + j * CPM; c < kLead + (j + 1) * CPM; ++c)
+                if (c < 16) prob2(c);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if constexpr (!kGeneral) {
+            // 2^24: some exponent exceeded the reference by more than ~19; also true for the
+            // first visible tile of a row (reference still "minus huge" -> infinite sum)
+            // The scores were given up register by register as the pairs consumed them, so
+            // this rare path first recomputes them, with K fragments straight from global
+            // memory (the tile's LDS buffer may already be in the hands of a faster wave).
+            if (__any(l_tile > 16777216.f)) {
+#pragma unroll
+                for (int sx = 0; sx < KS; ++sx)
 #pragma unroll
                     for (int kb = 0; kb < 2; ++kb) {
-                        if (g == 0 && t == 0) {
+                        const uint32_t row = src_row(n0 + kb * 32 + lq);
+                        const u32x4 a = *reinterpret_cast<const u32x4*>(
+                            kbase + (size_t)row * rb + (uint32_t)(16 * sx + 8 * lh) * 2u);
+                        if (sx == 0) {
                             floatx16 z;
 #pragma unroll
                             for (int i = 0; i < 16; ++i) z[i] = 0.f;
-                            snext[kb] = Ops::mfma(kf[t][kb], qf[0], z);
+                            scur[kb] = Ops::mfma(a, qf[0], z);
                         } else {
-                            snext[kb] = Ops::mfma(kf[t][kb], qf[g * SPS + t], snext[kb]);
+                            scur[kb] = Ops::mfma(a, qf[sx], scur[kb]);
                         }
                     }
-                prob4(g, 1);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            // 2^24: some exponent exceeded the reference by more than ~19; also true for the
-            // first visible tile of a row (reference still "minus huge" -> infinite sum)
-            if (__any(l_tile > 16777216.f)) {
                 rebase();
                 probabilities();
             }
         }
         l_run += l_tile;
 
-        // O^T += V^T P^T, V operands read one 16-key step ahead of their MFMAs
-        {
-            u32x4 vf[2][DB];
+        // O^T += V^T P^T.  In the shadow of these MFMAs the staging registers go to LDS --
+        // K(it+2) and V(it+1), into the buffers whose last readers finished before this step's
+        // barrier -- and are refilled with K(it+3) and V(it+2).
 #pragma unroll
-            for (int b = 0; b < DB; ++b) vf[0][b] = ksa_read_vt_frag<VROW>(Vs[it & 1], 0, b, lq, lh);
-#pragma unroll
-            for (int ks = 0; ks < 4; ++ks) {
-                if (ks < 3) {
-#pragma unroll
-                    for (int b = 0; b < DB; ++b)
-                        vf[(ks + 1) & 1][b] = ksa_read_vt_frag<VROW>(Vs[it & 1], ks + 1, b, lq, lh);
-                }
-#pragma unroll
-                for (int b = 0; b < DB; ++b) oacc[b] = Ops::mfma(vf[ks & 1][b], pf[ks], oacc[b]);
-                __builtin_amdgcn_sched_barrier(0);
-            }
+        for (int j = 0; j < NPV; ++j) {
+            oacc[j % DB] = Ops::mfma(fq[j % kQueue], pf[j / DB], oacc[j % DB]);
+            if (j + kQueue < NPV) fq[j % kQueue] = vfrag(j + kQueue);
+            if (j == 0) store_k(it & 1);
+            if (j == NPV / 4) store_v((it + 1) & 1);
+            if (j == NPV / 2) load_kv(kbase, kreg, nk, wk);
+            if (j == (3 * NPV) / 4) load_kv(vbase, vreg, nv, wv);
+            __builtin_amdgcn_sched_barrier(0);
         }
         if ((it & 63) == 63) {  // roll the index chunk
             seq_cur = seq_nxt;
@@ -456,13 +474,17 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
     };
 
     floatx16 s0[2], s1[2];
-    if (ntiles > 0) {  // prologue: scores of tile 0, then K(1) and V(0) into registers
+    if (ntiles > 0) {  // prologue: K(0), K(1), V(0) in LDS, scores of tile 0, K(2), V(1) in registers
+        const int i1 = min(1, ntiles - 1), i2 = min(2, ntiles - 1);
         load_kv(kbase, kreg, seq(0, 0), seq_word(0, 0));
-        store_k(0);
-        __syncthreads();
-        const int i1 = min(1, ntiles - 1);
-        load_kv(kbase, kreg, seq(i1, 0), seq_word(i1, 0));
         load_kv(vbase, vreg, seq(0, 0), seq_word(0, 0));
+        store_k(0);
+        store_v(0);
+        load_kv(kbase, kreg, seq(i1, 0), seq_word(i1, 0));
+        load_kv(vbase, vreg, seq(i1, 0), seq_word(i1, 0));
+        store_k(1);
+        __syncthreads();
+        load_kv(kbase, kreg, seq(i2, 0), seq_word(i2, 0));
         scores(s0, 0);
     }
     auto copy_scores = [&]() {
