@@ -27,6 +27,7 @@
 // 64-bit visibility word per query row.
 #include <hip/hip_runtime.h>
 #include <math.h>
+#include <stdlib.h>
 
 #include <type_traits>
 
@@ -56,6 +57,7 @@ struct PrefillParams {
     KsaMask mk;
     float scale;
     float scale_log2;
+    int rows_per_wave;  // 64: two row blocks per wave where the shape allows (experimental)
 };
 
 constexpr int kThreads = 256;
@@ -97,8 +99,15 @@ __device__ __forceinline__ RowVis ksa_row_vis(const KsaMask& mk, int q) {
 // kRegular: every listed key tile lies entirely in the summary prefix or entirely in the
 // in-line region and inside the key axis (P and Sk multiples of 64), and in-place prefix
 // rows of one thread differ by a uniform step; then tile addressing is branch-free.
-template <typename T, int D, bool kRegular>
-__global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillParams p) {
+//
+// RB: 32-row query blocks per wave.  RB = 1: one query head per workgroup, wave w owns rows
+// 32w..32w+31, two workgroups per CU.  RB = 2: two query heads of one kv group per workgroup,
+// waves {0,1} / {2,3} own rows 0..63 / 64..127 of the first / second head, one workgroup per
+// CU with up to 512 registers per lane; every K and V fragment read from LDS then feeds two
+// MFMAs, which halves the LDS traffic per MFMA (at one fragment per MFMA the four SIMDs ask
+// for more than the LDS delivers).
+template <typename T, int D, bool kRegular, int RB>
+__global__ __launch_bounds__(kThreads, (RB == 1 ? 2 : 1)) void ksa_prefill_kernel(const PrefillParams p) {
     using Ops = KsaOps<T>;
     constexpr int KS = D / 16;       // contraction steps of K Q^T
     constexpr int DB = D / 32;       // 32-row blocks of O^T
@@ -118,30 +127,34 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
     const int lq = lane & 31;
     const int lh = lane >> 5;
 
-    // workgroup -> (kv head, query head in group, m tile); kv head fastest so that
+    // workgroup -> (kv head, query head (pair) in group, m tile); kv head fastest so that
     // the workgroups sharing K/V land on one XCD; heavy (late) m tiles first.
     const int bz = blockIdx.y;
     const int id = blockIdx.x;
     const int kvh = id % p.Hkv;
     const int rest = id / p.Hkv;
-    const int gi = rest % p.g;
-    const int mt = p.M - 1 - rest / p.g;
-    const int head = kvh * p.g + gi;
+    const int gper = p.g / RB;
+    const int gi = rest % gper;
+    const int mt = p.M - 1 - rest / gper;
+    const int head = kvh * p.g + (RB == 1 ? gi : 2 * gi + (wave >> 1));
+    const int row0 = mt * kTileM + (RB == 1 ? wave * 32 : (wave & 1) * 64);
     const KsaMask mk = p.mk;
     const bool prefix_mode = mk.P > 0;
     const bool phys = p.phys_prefix != 0;
     const int Bblk = mk.C + mk.S;
 
-    const int qrow = mt * kTileM + wave * 32 + lq;
-    const int qrow_c = min(qrow, mk.Sq - 1);
-    const RowVis rv = ksa_row_vis(mk, qrow_c);
-
+    int qrow[RB];
+    RowVis rv[RB];
     // Q as B operand, resident in registers for the whole tile walk
-    u32x4 qf[KS];
-    {
+    u32x4 qf[RB][KS];
+#pragma unroll
+    for (int r = 0; r < RB; ++r) {
+        qrow[r] = row0 + 32 * r + lq;
+        const int qrow_c = min(qrow[r], mk.Sq - 1);
+        rv[r] = ksa_row_vis(mk, qrow_c);
         const uint16_t* qp = p.q + bz * p.q_bs + (int64_t)qrow_c * p.q_rs + head * p.q_hs + 8 * lh;
 #pragma unroll
-        for (int s = 0; s < KS; ++s) qf[s] = *reinterpret_cast<const u32x4*>(qp + 16 * s);
+        for (int s = 0; s < KS; ++s) qf[r][s] = *reinterpret_cast<const u32x4*>(qp + 16 * s);
     }
 
     // ---- K/V addressing: uniform base + uniform tile offset + 32-bit thread offset ----
@@ -167,9 +180,6 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
 
     // tile -> (uniform byte offset, uniform per-load step, per-thread byte offsets)
     auto tile_src = [&](int n0, uint32_t& ubase, uint32_t& ustep, uint32_t (&voff)[KLD]) {
-        if constexpr (kRegular) {  // not used: regular tiles take the precomputed offset word
-            (void)n0;
-        }
         const bool in_main = (phys || n0 >= mk.P) && n0 + kTileN <= mk.Sk;
         if (in_main) {
             ubase = (uint32_t)(phys ? n0 : n0 - mk.P) * rb;
@@ -215,15 +225,19 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
         for (int i = 0; i < KLD; ++i)
             reg[i] = *reinterpret_cast<const u32x4*>(base + (ub + us * i) + vo[i]);
     };
+    auto store_k1 = [&](int buf, int i) {
+        *reinterpret_cast<u32x4*>(&Ks[buf][(ld_row + RSTEP * i) * KROW + 8 * (tid % CPR)]) = kreg[i];
+    };
+    auto store_v1 = [&](int buf, int i) {
+        *reinterpret_cast<u32x4*>(&Vs[buf][(ld_row + RSTEP * i) * VROW + 8 * (tid % CPR)]) = vreg[i];
+    };
     auto store_k = [&](int buf) {
 #pragma unroll
-        for (int i = 0; i < KLD; ++i)
-            *reinterpret_cast<u32x4*>(&Ks[buf][(ld_row + RSTEP * i) * KROW + 8 * (tid % CPR)]) = kreg[i];
+        for (int i = 0; i < KLD; ++i) store_k1(buf, i);
     };
     auto store_v = [&](int buf) {
 #pragma unroll
-        for (int i = 0; i < KLD; ++i)
-            *reinterpret_cast<u32x4*>(&Vs[buf][(ld_row + RSTEP * i) * VROW + 8 * (tid % CPR)]) = vreg[i];
+        for (int i = 0; i < KLD; ++i) store_v1(buf, i);
     };
 
     // ---- walk order ----
@@ -262,7 +276,7 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
     int seq_nxt = seq_chunk(64);
     uint32_t word_cur = kRegular ? tile_word(seq_cur) : 0u;
     uint32_t word_nxt = kRegular ? tile_word(seq_nxt) : 0u;
-    // entry i in {it, it+1, it+2} while processing tile it
+    // entry i in {it, .., it+3} while processing tile it
     auto seq = [&](int i, int it) {
         const int src = (i >> 6) == (it >> 6) ? seq_cur : seq_nxt;
         return __builtin_amdgcn_readlane(src, i & 63);
@@ -272,40 +286,59 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
         return (uint32_t)__builtin_amdgcn_readlane((int)src, i & 63);
     };
 
-    floatx16 oacc[DB];
-#pragma unroll
-    for (int b = 0; b < DB; ++b)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) oacc[b][i] = 0.f;
+    floatx16 oacc[RB][DB];
     // reference maximum of the exponents (raw score units); a finite "minus huge" start
     // value makes the first visible tile rescale the (still zero) accumulators by 0
-    float m_ref = -1e30f;
-    float l_run = 0.f;        // this lane's half of the row sum
+    float m_ref[RB];
+    float l_run[RB];  // this lane's half of the row sum
+#pragma unroll
+    for (int r = 0; r < RB; ++r) {
+        m_ref[r] = -1e30f;
+        l_run[r] = 0.f;
+#pragma unroll
+        for (int b = 0; b < DB; ++b)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) oacc[r][b][i] = 0.f;
+    }
     const float c2 = p.scale_log2;
 
-    auto scores = [&](floatx16 (&sacc)[2], int buf) {  // S^T = K Q^T for the tile in Ks[buf]
+    auto zero16 = []() {
+        floatx16 z;
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) sacc[kb][i] = 0.f;
+        for (int i = 0; i < 16; ++i) z[i] = 0.f;
+        return z;
+    };
+
+    auto scores = [&](floatx16 (&sacc)[RB][2], int buf) {  // S^T = K Q^T for the tile in Ks[buf]
 #pragma unroll
         for (int s = 0; s < KS; ++s) {
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb) {
                 const u32x4 a = *reinterpret_cast<const u32x4*>(
                     &Ks[buf][(kb * 32 + lq) * KROW + 16 * s + 8 * lh]);
-                sacc[kb] = Ops::mfma(a, qf[s], sacc[kb]);
+#pragma unroll
+                for (int r = 0; r < RB; ++r) {
+                    if constexpr (RB == 1) {
+                        sacc[r][kb] = Ops::mfma(a, qf[r][s], s == 0 ? zero16() : sacc[r][kb]);
+                    } else {
+                        if (s == 0) sacc[r][kb] = Ops::mfma_v0(a, qf[r][s]);
+                        else Ops::mfma_v(sacc[r][kb], a, qf[r][s]);
+                    }
+                }
             }
         }
+        if constexpr (RB != 1) ksa_mfma_settle();
     };
 
     // One pipeline step for tile `it`: its scores are in `scur`; the scores of tile it+1
     // are produced into `snext`.  On entry LDS holds (or is being written with) K(it+1) and
     // V(it), and the registers hold K(it+2) and V(it+1).  The barrier publishes the LDS tiles;
-    // the staging registers are written to the buffers freed by the previous step and refilled
-    // from global memory in the shadow of the second product's MFMAs, so that no wave ever
-    // sits in a block of loads or LDS stores with the matrix unit idle.
-    auto step = [&](auto general_tag, int it, floatx16 (&scur)[2], floatx16 (&snext)[2], bool row_vis) {
+    // the staging registers are written to the buffers freed by the previous step in the
+    // shadow of the score MFMAs and refilled from global memory in the shadow of the second
+    // product's, so that no wave ever sits in a block of loads or LDS stores with the matrix
+    // unit idle.
+    // `quick`: a row is visible as a whole iff it is a text row (leading prefix tiles).
+    auto step = [&](auto general_tag, int it, floatx16 (&scur)[RB][2], floatx16 (&snext)[RB][2], bool quick) {
         constexpr bool kGeneral = decltype(general_tag)::value;
         const int n0 = seq(it, it) * kTileN;
         // Past the end of the walk the pipeline keeps running on the last tile (loads) and
@@ -313,15 +346,19 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
         const int ik = min(it + 3, ntiles - 1), iv = min(it + 2, ntiles - 1);
         const int nk = seq(ik, it), nv = seq(iv, it);
         const uint32_t wk = seq_word(ik, it), wv = seq_word(iv, it);
+        bool row_vis[RB];
+#pragma unroll
+        for (int r = 0; r < RB; ++r) row_vis[r] = quick ? rv[r].b_text : true;
         __syncthreads();
 
         // MFMA operands that come from LDS travel through a rolling queue of kQueue fragments:
-        // the read for operand j + kQueue is issued right behind MFMA j, through the score
-        // product (K fragments), across its end (the first V fragments) and through the second
-        // product, so every read has kQueue MFMAs plus the vector work between them to land.
+        // the read for operand j + kQueue is issued right behind the MFMAs of operand j, through
+        // the score product (K fragments), across its end (the first V fragments) and through
+        // the second product, so every read has kQueue operands' worth of MFMAs plus the vector
+        // work between them to land.
         constexpr int kQueue = 4;
-        constexpr int NQK = 2 * KS;   // score MFMAs: contraction step s = j / 2, key block kb = j % 2
-        constexpr int NPV = 4 * DB;   // second-product MFMAs: key step ks = j / DB, dim block j % DB
+        constexpr int NQK = 2 * KS;   // K fragments: contraction step s = j / 2, key block kb = j % 2
+        constexpr int NPV = 4 * DB;   // V fragments: key step ks = j / DB, dim block j % DB
         const uint16_t* ksrc = Ks[(it + 1) & 1];
         const uint16_t* vsrc = Vs[it & 1];
         auto kfrag = [&](int j) {
@@ -340,16 +377,19 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
             const uint64_t valid = __ballot(in);
             const uint64_t text = __ballot(in && rel >= 0 && (rel % Bblk) < mk.C);
             const uint64_t fa = prefix_mode ? valid : (valid & ~text);
-            const uint64_t fb = rv.b_text ? text : valid;
-            const uint64_t bits = (ksa_range_bits(-n0, rv.xa - n0) & fa) |
-                                  (ksa_range_bits(rv.blo - n0, rv.bhi - n0) & fb);
-            const uint64_t sh = bits >> (4 * lh);
-            const uint32_t w0 = (uint32_t)sh, w1 = (uint32_t)(sh >> 32);
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const uint32_t bit = 1u << (8 * (i / 4) + (i % 4));
-                scur[0][i] = (w0 & bit) ? scur[0][i] : -INFINITY;
-                scur[1][i] = (w1 & bit) ? scur[1][i] : -INFINITY;
+            for (int r = 0; r < RB; ++r) {
+                const uint64_t fb = rv[r].b_text ? text : valid;
+                const uint64_t bits = (ksa_range_bits(-n0, rv[r].xa - n0) & fa) |
+                                      (ksa_range_bits(rv[r].blo - n0, rv[r].bhi - n0) & fb);
+                const uint64_t sh = bits >> (4 * lh);
+                const uint32_t w0 = (uint32_t)sh, w1 = (uint32_t)(sh >> 32);
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const uint32_t bit = 1u << (8 * (i / 4) + (i % 4));
+                    scur[r][0][i] = (w0 & bit) ? scur[r][0][i] : -INFINITY;
+                    scur[r][1][i] = (w1 & bit) ? scur[r][1][i] : -INFINITY;
+                }
             }
         }
 
@@ -357,79 +397,144 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
         // only where it is needed: always on the masked tiles of phase B; on phase A tiles
         // only after the fact, when a row has no reference yet or its tile sum shows that the
         // exponents outgrew the reference (then the tile's probabilities are redone).
-        float l_tile = 0.f;
-        u32x4 pf[4];
-        float mc = row_vis ? m_ref * c2 : INFINITY;
-        // probability pair c (0..15): keys of 16-key group c / 4, packed word c % 4
-        auto prob2 = [&](int c) {
+        float l_tile[RB];
+        u32x4 pf[RB][4];
+        float mc[RB];
+#pragma unroll
+        for (int r = 0; r < RB; ++r) {
+            l_tile[r] = 0.f;
+            mc[r] = row_vis[r] ? m_ref[r] * c2 : INFINITY;
+        }
+        // Probability pair cc (row block cc / 16, keys of 16-key group (cc % 16) / 4, word cc % 4)
+        // in four dependent stages.  In the interleaved loop below the stages of one pair run
+        // in consecutive time slots, so no vector instruction waits for its predecessor.
+        float pa[2][2];
+        uint32_t pw[2];
+        auto stage_a = [&](int cc) {  // exponent arguments
+            const int r = cc >> 4, c = cc & 15;
             const int g = c >> 2, kb = g >> 1, i0 = 8 * (g & 1) + 2 * (c & 3);
-            const float p0 = ksa_exp2(fmaf(scur[kb][i0], c2, -mc));
-            const float p1 = ksa_exp2(fmaf(scur[kb][i0 + 1], c2, -mc));
-            const uint32_t pk = Ops::pack2(p0, p1);
-            l_tile = Ops::sum2(pk, l_tile);
-            pf[g][c & 3] = pk;
+            pa[cc & 1][0] = fmaf(scur[r][kb][i0], c2, -mc[r]);
+            pa[cc & 1][1] = fmaf(scur[r][kb][i0 + 1], c2, -mc[r]);
+        };
+        auto stage_b = [&](int cc) {
+            pa[cc & 1][0] = ksa_exp2(pa[cc & 1][0]);
+            pa[cc & 1][1] = ksa_exp2(pa[cc & 1][1]);
+        };
+        auto stage_c = [&](int cc) { pw[cc & 1] = Ops::pack2(pa[cc & 1][0], pa[cc & 1][1]); };
+        auto stage_d = [&](int cc) {
+            const int r = cc >> 4, c = cc & 15;
+            l_tile[r] = Ops::sum2(pw[cc & 1], l_tile[r]);
+            pf[r][c >> 2][c & 3] = pw[cc & 1];
+        };
+        constexpr int NCH = 16 * RB;
+        // time slot vt: stage d of pair vt-3, c of vt-2, b of vt-1, a of vt
+        auto prob_slot = [&](int vt) {
+            if (vt >= 3 && vt - 3 < NCH) stage_d(vt - 3);
+            if (vt >= 2 && vt - 2 < NCH) stage_c(vt - 2);
+            if (vt >= 1 && vt - 1 < NCH) stage_b(vt - 1);
+            if (vt < NCH) stage_a(vt);
+        };
+        auto prob2 = [&](int cc) {
+            stage_a(cc);
+            stage_b(cc);
+            stage_c(cc);
+            stage_d(cc);
         };
         auto probabilities = [&]() {
-            mc = row_vis ? m_ref * c2 : INFINITY;
-            l_tile = 0.f;
 #pragma unroll
-            for (int c = 0; c < 16; ++c) prob2(c);
+            for (int r = 0; r < RB; ++r) {
+                mc[r] = row_vis[r] ? m_ref[r] * c2 : INFINITY;
+                l_tile[r] = 0.f;
+            }
+#pragma unroll
+            for (int cc = 0; cc < 16 * RB; ++cc) prob2(cc);
         };
         // move the reference of the rows whose maximum outgrew it (or that have none yet)
         auto rebase = [&]() {
-            float mloc = fmaxf(scur[0][0], scur[1][0]);
 #pragma unroll
-            for (int i = 1; i < 16; ++i) mloc = fmaxf(mloc, fmaxf(scur[0][i], scur[1][i]));
-            if (!row_vis) mloc = -INFINITY;
-            mloc = ksa_pair_max(mloc);
-            const bool bump = (mloc - m_ref) * c2 > kTau;
-            if (__any(bump)) {
-                const float m_new = bump ? mloc : m_ref;
-                const float alpha = ksa_exp2((m_ref - m_new) * c2);
-                m_ref = m_new;
-                l_run *= alpha;
+            for (int r = 0; r < RB; ++r) {
+                float mloc = fmaxf(scur[r][0][0], scur[r][1][0]);
 #pragma unroll
-                for (int b = 0; b < DB; ++b)
+                for (int i = 1; i < 16; ++i) mloc = fmaxf(mloc, fmaxf(scur[r][0][i], scur[r][1][i]));
+                if (!row_vis[r]) mloc = -INFINITY;
+                mloc = ksa_pair_max(mloc);
+                const bool bump = (mloc - m_ref[r]) * c2 > kTau;
+                if (__any(bump)) {
+                    const float m_new = bump ? mloc : m_ref[r];
+                    const float alpha = ksa_exp2((m_ref[r] - m_new) * c2);
+                    m_ref[r] = m_new;
+                    l_run[r] *= alpha;
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) oacc[b][i] *= alpha;
+                    for (int b = 0; b < DB; ++b) {
+#pragma unroll
+                        for (int i = 0; i < 16; ++i) oacc[r][b][i] *= alpha;
+                        if constexpr (RB != 1) {
+                            // back to its AGPR block before the next one is touched, so that
+                            // this rare path never holds more than one block in VGPRs
+                            asm volatile("" : "+a"(oacc[r][b]));
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                    }
+                }
             }
         };
         if constexpr (kGeneral) {
             rebase();
-            mc = row_vis ? m_ref * c2 : INFINITY;
+#pragma unroll
+            for (int r = 0; r < RB; ++r) mc[r] = row_vis[r] ? m_ref[r] * c2 : INFINITY;
         }
 
         // Score MFMAs of the NEXT tile with the probability pairs of THIS tile between them.
-        // The fences pin the order; kLead pairs run first and cover the first operand reads.
+        // The fences pin the order; kLead slots run first and cover the first operand reads.
+        // The second half of the loop also carries the LDS stores of the staging registers:
+        // K(it+2) and V(it+1) go to the buffers whose last readers finished before this step's
+        // barrier (the LDS queue of a wave is idle here and saturated in the second product).
         constexpr int CPM = 16 / NQK;            // probability pairs per score MFMA
-        constexpr int kLead = 3 * CPM;
+        constexpr int kLead = 3;
+        constexpr int NM = NQK * RB;
+        constexpr int kStoreStep = (NM / 2) / (2 * KLD);
+        static_assert(kStoreStep >= 1, "one LDS store per MFMA slot at most");
 #pragma unroll
-        for (int c = 0; c < kLead; ++c) prob2(c);
+        for (int vt = 0; vt < kLead; ++vt) prob_slot(vt);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int j = 0; j < NQK; ++j) {
             const int kb = j & 1;
-            if (j < 2) {
-                floatx16 z;
 #pragma unroll
-                for (int i = 0; i < 16; ++i) z[i] = 0.f;
-                snext[kb] = Ops::mfma(fq[j % kQueue], qf[0], z);
-            } else {
-                snext[kb] = Ops::mfma(fq[j % kQueue], qf[j >> 1], snext[kb]);
+            for (int r = 0; r < RB; ++r) {
+                if constexpr (RB == 1) {
+                    snext[r][kb] = Ops::mfma(fq[j % kQueue], qf[r][j >> 1], j < 2 ? zero16() : snext[r][kb]);
+                } else {
+                    if (j < 2) snext[r][kb] = Ops::mfma_v0(fq[j % kQueue], qf[r][j >> 1]);
+                    else Ops::mfma_v(snext[r][kb], fq[j % kQueue], qf[r][j >> 1]);
+                }
+                if (r == RB - 1)
+                    fq[j % kQueue] = (j + kQueue < NQK) ? kfrag(j + kQueue) : vfrag(j + kQueue - NQK);
+                const int m = j * RB + r;
+#pragma unroll
+                for (int vt = kLead + m * CPM; vt < kLead + (m + 1) * CPM; ++vt) prob_slot(vt);
+                if (m >= NM / 2 && (m - NM / 2) % kStoreStep == 0) {
+                    const int si = (m - NM / 2) / kStoreStep;
+                    if (si < KLD) store_k1(it & 1, si);
+                    else if (si < 2 * KLD) store_v1((it + 1) & 1, si - KLD);
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
-            fq[j % kQueue] = (j + kQueue < NQK) ? kfrag(j + kQueue) : vfrag(j + kQueue - NQK);
-#pragma unroll
-            for (int c = kLead + j * CPM; c < kLead + (j + 1) * CPM; ++c)
-                if (c < 16) prob2(c);
-            __builtin_amdgcn_sched_barrier(0);
         }
         if constexpr (!kGeneral) {
             // 2^24: some exponent exceeded the reference by more than ~19; also true for the
-            // first visible tile of a row (reference still "minus huge" -> infinite sum)
+            // first visible tile of a row (reference still "minus huge" -> infinite sum).
             // The scores were given up register by register as the pairs consumed them, so
             // this rare path first recomputes them, with K fragments straight from global
             // memory (the tile's LDS buffer may already be in the hands of a faster wave).
-            if (__any(l_tile > 16777216.f)) {
+            bool redo = false;
+#pragma unroll
+            for (int r = 0; r < RB; ++r) redo = redo || l_tile[r] > 16777216.f;
+#ifdef KSA_X_NOREDO
+            if (false) {
+#else
+            if (__any(redo)) {
+#endif
 #pragma unroll
                 for (int sx = 0; sx < KS; ++sx)
 #pragma unroll
@@ -437,32 +542,35 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
                         const uint32_t row = src_row(n0 + kb * 32 + lq);
                         const u32x4 a = *reinterpret_cast<const u32x4*>(
                             kbase + (size_t)row * rb + (uint32_t)(16 * sx + 8 * lh) * 2u);
-                        if (sx == 0) {
-                            floatx16 z;
 #pragma unroll
-                            for (int i = 0; i < 16; ++i) z[i] = 0.f;
-                            scur[kb] = Ops::mfma(a, qf[0], z);
-                        } else {
-                            scur[kb] = Ops::mfma(a, qf[sx], scur[kb]);
+                        for (int r = 0; r < RB; ++r) {
+                            if constexpr (RB == 1) {
+                                scur[r][kb] = Ops::mfma(a, qf[r][sx], sx == 0 ? zero16() : scur[r][kb]);
+                            } else {
+                                if (sx == 0) scur[r][kb] = Ops::mfma_v0(a, qf[r][sx]);
+                                else Ops::mfma_v(scur[r][kb], a, qf[r][sx]);
+                            }
                         }
                     }
+                if constexpr (RB != 1) ksa_mfma_settle();
                 rebase();
                 probabilities();
             }
         }
-        l_run += l_tile;
+#pragma unroll
+        for (int r = 0; r < RB; ++r) l_run[r] += l_tile[r];
 
-        // O^T += V^T P^T.  In the shadow of these MFMAs the staging registers go to LDS --
-        // K(it+2) and V(it+1), into the buffers whose last readers finished before this step's
-        // barrier -- and are refilled with K(it+3) and V(it+2).
+        // O^T += V^T P^T; the staging registers are refilled with K(it+3) and V(it+2).
 #pragma unroll
         for (int j = 0; j < NPV; ++j) {
-            oacc[j % DB] = Ops::mfma(fq[j % kQueue], pf[j / DB], oacc[j % DB]);
+#pragma unroll
+            for (int r = 0; r < RB; ++r) {
+                if constexpr (RB == 1) oacc[r][j % DB] = Ops::mfma(fq[j % kQueue], pf[r][j / DB], oacc[r][j % DB]);
+                else Ops::mfma_a(oacc[r][j % DB], fq[j % kQueue], pf[r][j / DB]);
+            }
             if (j + kQueue < NPV) fq[j % kQueue] = vfrag(j + kQueue);
-            if (j == 0) store_k(it & 1);
-            if (j == NPV / 4) store_v((it + 1) & 1);
-            if (j == NPV / 2) load_kv(kbase, kreg, nk, wk);
-            if (j == (3 * NPV) / 4) load_kv(vbase, vreg, nv, wv);
+            if (j == 0) load_kv(kbase, kreg, nk, wk);
+            if (j == NPV / 4) load_kv(vbase, vreg, nv, wv);
             __builtin_amdgcn_sched_barrier(0);
         }
         if ((it & 63) == 63) {  // roll the index chunk
@@ -473,7 +581,7 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
         }
     };
 
-    floatx16 s0[2], s1[2];
+    floatx16 s0[RB][2], s1[RB][2];
     if (ntiles > 0) {  // prologue: K(0), K(1), V(0) in LDS, scores of tile 0, K(2), V(1) in registers
         const int i1 = min(1, ntiles - 1), i2 = min(2, ntiles - 1);
         load_kv(kbase, kreg, seq(0, 0), seq_word(0, 0));
@@ -489,58 +597,75 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_prefill_kernel(const PrefillP
     }
     auto copy_scores = [&]() {
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
+        for (int r = 0; r < RB; ++r)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) s0[kb][i] = s1[kb][i];
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) s0[r][kb][i] = s1[r][kb][i];
     };
-    const bool lane_is_text = rv.b_text;
     int it = 0;
     for (; it + 2 <= n_a; it += 2) {
-        step(std::false_type{}, it, s0, s1, it < nquick ? lane_is_text : true);
-        step(std::false_type{}, it + 1, s1, s0, it + 1 < nquick ? lane_is_text : true);
+        step(std::false_type{}, it, s0, s1, it < nquick);
+        step(std::false_type{}, it + 1, s1, s0, it + 1 < nquick);
     }
     if (it < n_a) {
-        step(std::false_type{}, it, s0, s1, it < nquick ? lane_is_text : true);
+        step(std::false_type{}, it, s0, s1, it < nquick);
         copy_scores();
         ++it;
     }
     for (; it + 2 <= ntiles; it += 2) {
-        step(std::true_type{}, it, s0, s1, true);
-        step(std::true_type{}, it + 1, s1, s0, true);
+        step(std::true_type{}, it, s0, s1, false);
+        step(std::true_type{}, it + 1, s1, s0, false);
     }
-    if (it < ntiles) step(std::true_type{}, it, s0, s1, true);
+    if (it < ntiles) step(std::true_type{}, it, s0, s1, false);
 
     // ---- epilogue ----
-    const float l_tot = ksa_pair_sum(l_run);
-    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-    if (qrow < mk.Sq) {
-        uint16_t* op = p.out + bz * p.o_bs + (int64_t)qrow * p.o_rs + head * p.o_hs;
+    if constexpr (RB != 1) ksa_mfma_settle();
 #pragma unroll
-        for (int b = 0; b < DB; ++b)
+    for (int r = 0; r < RB; ++r) {
+        const float l_tot = ksa_pair_sum(l_run[r]);
+        const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+        if (qrow[r] < mk.Sq) {
+            uint16_t* op = p.out + bz * p.o_bs + (int64_t)qrow[r] * p.o_rs + head * p.o_hs;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                u32x2 w;
-                w[0] = Ops::pack2(oacc[b][4 * j] * inv, oacc[b][4 * j + 1] * inv);
-                w[1] = Ops::pack2(oacc[b][4 * j + 2] * inv, oacc[b][4 * j + 3] * inv);
-                *reinterpret_cast<u32x2*>(op + 32 * b + 8 * j + 4 * lh) = w;
-            }
-        if (p.lse && lh == 0)
-            p.lse[bz * p.lse_bs + head * p.lse_hs + qrow] =
-                l_tot > 0.f ? m_ref * p.scale + logf(l_tot) : -INFINITY;
+            for (int b = 0; b < DB; ++b)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    u32x2 w;
+                    w[0] = Ops::pack2(oacc[r][b][4 * j] * inv, oacc[r][b][4 * j + 1] * inv);
+                    w[1] = Ops::pack2(oacc[r][b][4 * j + 2] * inv, oacc[r][b][4 * j + 3] * inv);
+                    *reinterpret_cast<u32x2*>(op + 32 * b + 8 * j + 4 * lh) = w;
+                }
+            if (p.lse && lh == 0)
+                p.lse[bz * p.lse_bs + head * p.lse_hs + qrow[r]] =
+                    l_tot > 0.f ? m_ref[r] * p.scale + logf(l_tot) : -INFINITY;
+        }
     }
 }
 
 template <typename T, int D>
 int launch(const PrefillParams& p, int batch, hipStream_t stream) {
-    dim3 grid(p.M * p.Hq, batch);
     constexpr int RSTEP = kThreads / (D / 8);
     const KsaMask& mk = p.mk;
     const bool prefix_ok = mk.P == 0 || p.phys_prefix || (RSTEP % mk.S == 0 && mk.P % kTileN == 0);
     const bool regular = prefix_ok && mk.Sk % kTileN == 0;
-    if (regular)
-        hipLaunchKernelGGL((ksa_prefill_kernel<T, D, true>), grid, dim3(kThreads), 0, stream, p);
-    else
-        hipLaunchKernelGGL((ksa_prefill_kernel<T, D, false>), grid, dim3(kThreads), 0, stream, p);
+    // two heads per workgroup need an even group size; the wider kernel is built for D = 128
+    const bool pair = D == 128 && p.g % 2 == 0 && p.rows_per_wave == 64;
+    if (pair) {
+        dim3 grid(p.M * (p.Hq / 2), batch);
+        if constexpr (D == 128) {
+            if (regular)
+                hipLaunchKernelGGL((ksa_prefill_kernel<T, D, true, 2>), grid, dim3(kThreads), 0, stream, p);
+            else
+                hipLaunchKernelGGL((ksa_prefill_kernel<T, D, false, 2>), grid, dim3(kThreads), 0, stream, p);
+        }
+    } else {
+        dim3 grid(p.M * p.Hq, batch);
+        if (regular)
+            hipLaunchKernelGGL((ksa_prefill_kernel<T, D, true, 1>), grid, dim3(kThreads), 0, stream, p);
+        else
+            hipLaunchKernelGGL((ksa_prefill_kernel<T, D, false, 1>), grid, dim3(kThreads), 0, stream, p);
+    }
     return ksa_check_launch();
 }
 
@@ -602,6 +727,10 @@ extern "C" int ksa_prefill_fwd(const void* q, const void* k, const void* v, void
     p.mk = KsaMask{C, S, W, P, skip_old ? 1 : 0, Sq, Sk};
     p.scale = scale;
     p.scale_log2 = scale * 1.4426950408889634f;
+    // KSA_PREFILL_ROWS_PER_WAVE=64 selects the two-head workgroup (64 query rows per wave, one
+    // wave per SIMD) where the shape allows; it is correct but not yet faster
+    const char* rpw = getenv("KSA_PREFILL_ROWS_PER_WAVE");
+    p.rows_per_wave = rpw ? atoi(rpw) : 0;
 
     hipStream_t st = (hipStream_t)stream;
     if (dtype == KSA_DTYPE_BF16) {

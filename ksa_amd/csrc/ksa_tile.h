@@ -40,6 +40,22 @@ struct KsaOps<KsaBf16> {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
                                                        __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
     }
+    // Register-class pinned forms for kernels that run one wave per SIMD with both register
+    // files: accumulators of the second product (`acc`) and the resident B operand of the
+    // first (`b_acc`) live in AGPRs, scores and LDS-fed operands in VGPRs.  The compiler does
+    // not see an MFMA in these statements, so the caller keeps MFMA results away from vector
+    // instructions for the required wait states (ksa_mfma_settle).
+    static __device__ __forceinline__ floatx16 mfma_v0(u32x4 a, u32x4 b_acc) {
+        floatx16 d;
+        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "a"(b_acc));
+        return d;
+    }
+    static __device__ __forceinline__ void mfma_v(floatx16& c, u32x4 a, u32x4 b_acc) {
+        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b_acc));
+    }
+    static __device__ __forceinline__ void mfma_a(floatx16& acc, u32x4 a, u32x4 b) {
+        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+    }
     static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
         bf16x2 v;
         v[0] = (__bf16)lo;
@@ -60,6 +76,17 @@ struct KsaOps<KsaF16> {
     static __device__ __forceinline__ floatx16 mfma(u32x4 a, u32x4 b, floatx16 c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
                                                       __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ floatx16 mfma_v0(u32x4 a, u32x4 b_acc) {
+        floatx16 d;
+        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "a"(b_acc));
+        return d;
+    }
+    static __device__ __forceinline__ void mfma_v(floatx16& c, u32x4 a, u32x4 b_acc) {
+        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b_acc));
+    }
+    static __device__ __forceinline__ void mfma_a(floatx16& acc, u32x4 a, u32x4 b) {
+        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
     }
     static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
         f16x2 v;
@@ -95,6 +122,11 @@ __device__ __forceinline__ u32x4 ksa_read_vt_frag(const uint16_t* vs, int ks, in
     r[3] = h2[1];
     return r;
 }
+
+// Wait states between an MFMA written as inline assembly and the first vector or memory
+// instruction that touches its result (the hardware does not interlock these; 8-pass MFMAs
+// need 11, this leaves a wide margin).
+__device__ __forceinline__ void ksa_mfma_settle() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
 
 __device__ __forceinline__ float ksa_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
