@@ -111,15 +111,25 @@ __global__ __launch_bounds__(kThreads, (RB == 1 ? 2 : 1)) void ksa_prefill_kerne
     using Ops = KsaOps<T>;
     constexpr int KS = D / 16;       // contraction steps of K Q^T
     constexpr int DB = D / 32;       // 32-row blocks of O^T
-    constexpr int KROW = D + 8;      // padded LDS row of K (elements)
-    constexpr int VROW = D + 32;     // padded LDS row of V (stride = 16 banks mod 64)
     constexpr int CPR = D / 8;       // 16-byte chunks per K/V row
+    constexpr int ROWB = 2 * D;      // LDS row of K / V in bytes (unpadded, XOR-swizzled chunks)
     constexpr int KLD = (kTileN * CPR) / kThreads;  // K (and V) loads per thread
     constexpr int RSTEP = kThreads / CPR;           // row distance between a thread's loads
     constexpr float kTau = 8.f;      // lazy rescale: exponents stay below 2^kTau
 
-    __shared__ __attribute__((aligned(16))) uint16_t Ks[2][kTileN * KROW];
-    __shared__ __attribute__((aligned(16))) uint16_t Vs[2][kTileN * VROW];
+    // K and V tiles travel global -> LDS directly (global_load_lds), 1 KB per wave
+    // instruction, so LDS rows cannot be padded; bank conflicts are avoided by permuting the
+    // 16-byte chunks inside each row instead:
+    //   K: chunk c of tile row r sits at position c ^ ksw(r)  (the 16 lanes of a b128 read
+    //      phase hold 16 consecutive rows and the same chunk)
+    //   V: 64-byte segment s of row r sits at segment s ^ vsw(r)  (a transposing b64 read
+    //      phase covers 4 consecutive rows and one segment)
+    // Four separate arrays (not one [2][..]) so that the compiler can tell the buffer being
+    // filled from the one being read and does not wait for the fill before unrelated reads.
+    __shared__ __attribute__((aligned(1024))) uint16_t Ks0[kTileN * D];
+    __shared__ __attribute__((aligned(1024))) uint16_t Ks1[kTileN * D];
+    __shared__ __attribute__((aligned(1024))) uint16_t Vs0[kTileN * D];
+    __shared__ __attribute__((aligned(1024))) uint16_t Vs1[kTileN * D];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -162,13 +172,18 @@ __global__ __launch_bounds__(kThreads, (RB == 1 ? 2 : 1)) void ksa_prefill_kerne
     const char* vbase = reinterpret_cast<const char*>(p.v + bz * p.kv_bs + kvh * p.kv_hs);
     const uint32_t rb = (uint32_t)p.kv_rs * 2u;  // row pitch in bytes
     const int ld_row = tid / CPR;                // first tile row this thread loads
-    const uint32_t ld_col = (uint32_t)(tid % CPR) * 16u;
-    const uint32_t thr_main = (uint32_t)ld_row * rb + ld_col;
+    auto ksw = [](int r) { return D == 128 ? (r & 15) : ((r >> 1) & 7); };
+    auto vsw = [](int r) { return D == 128 ? (r & 3) : ((r >> 1) & 1); };
+    // this thread fills chunk position tid % CPR of its rows: the source chunk is the position
+    // with the row's permutation undone (rows of one thread differ by multiples of 16 or 32)
+    const uint32_t kcol = (uint32_t)((tid % CPR) ^ ksw(ld_row)) * 16u;
+    const uint32_t vcol = (uint32_t)((tid % CPR) ^ (vsw(ld_row) << 2)) * 16u;
+    const uint32_t thr_main = (uint32_t)ld_row * rb;
     // in-place prefix: prefix row j lives at in-line row (j / S) * B + C + j % S; when S
     // divides the per-thread row step the rows of one thread differ by a uniform amount
     const bool s_fast = !phys && (RSTEP % mk.S == 0);
     const uint32_t thr_pre =
-        s_fast ? (uint32_t)((ld_row / mk.S) * Bblk + mk.C + ld_row % mk.S) * rb + ld_col : 0u;
+        s_fast ? (uint32_t)((ld_row / mk.S) * Bblk + mk.C + ld_row % mk.S) * rb : 0u;
     const uint32_t step_main = RSTEP * rb;
     const uint32_t step_pre = s_fast ? (uint32_t)(RSTEP / mk.S) * Bblk * rb : 0u;
 
@@ -195,7 +210,7 @@ __global__ __launch_bounds__(kThreads, (RB == 1 ? 2 : 1)) void ksa_prefill_kerne
             ubase = 0;
             ustep = 0;
 #pragma unroll
-            for (int i = 0; i < KLD; ++i) voff[i] = src_row(n0 + ld_row + RSTEP * i) * rb + ld_col;
+            for (int i = 0; i < KLD; ++i) voff[i] = src_row(n0 + ld_row + RSTEP * i) * rb;
         }
     };
 
@@ -207,9 +222,9 @@ __global__ __launch_bounds__(kThreads, (RB == 1 ? 2 : 1)) void ksa_prefill_kerne
         return in_main ? ((uint32_t)(phys ? n0 : n0 - mk.P) * rb) | 1u
                        : (uint32_t)(n0 / mk.S) * Bblk * rb;
     };
-    u32x4 kreg[KLD];
-    u32x4 vreg[KLD];
-    auto load_kv = [&](const char* base, u32x4 (&reg)[KLD], int n, uint32_t word) {
+    // one 1 KB piece (load i of KLD) of tile n into an LDS tile; `col` = kcol or vcol
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    auto fill1 = [&](const char* base, uint16_t* tile, uint32_t col, int n, uint32_t word, int i) {
         uint32_t ub, us, vo[KLD];
         if constexpr (kRegular) {
             const bool in_main = word & 1u;
@@ -217,27 +232,47 @@ __global__ __launch_bounds__(kThreads, (RB == 1 ? 2 : 1)) void ksa_prefill_kerne
             us = in_main ? step_main : step_pre;
             const uint32_t t = in_main ? thr_main : thr_pre;
 #pragma unroll
-            for (int i = 0; i < KLD; ++i) vo[i] = t;
+            for (int x = 0; x < KLD; ++x) vo[x] = t;
         } else {
             tile_src(n * kTileN, ub, us, vo);
         }
+        typedef __attribute__((address_space(1))) void* gptr;
+        typedef __attribute__((address_space(3))) void* lptr;
+        char* dst = reinterpret_cast<char*>(tile) + (RSTEP * i + wave_u * (64 / CPR)) * ROWB;
+        __builtin_amdgcn_global_load_lds((gptr)(base + (ub + us * i) + vo[i] + col), (lptr)dst, 16, 0, 0);
+    };
+    auto fill = [&](const char* base, uint16_t* tile, uint32_t col, int n, uint32_t word) {
 #pragma unroll
-        for (int i = 0; i < KLD; ++i)
-            reg[i] = *reinterpret_cast<const u32x4*>(base + (ub + us * i) + vo[i]);
+        for (int i = 0; i < KLD; ++i) fill1(base, tile, col, n, word, i);
     };
-    auto store_k1 = [&](int buf, int i) {
-        *reinterpret_cast<u32x4*>(&Ks[buf][(ld_row + RSTEP * i) * KROW + 8 * (tid % CPR)]) = kreg[i];
-    };
-    auto store_v1 = [&](int buf, int i) {
-        *reinterpret_cast<u32x4*>(&Vs[buf][(ld_row + RSTEP * i) * VROW + 8 * (tid % CPR)]) = vreg[i];
-    };
-    auto store_k = [&](int buf) {
+    // all of this wave's fills have landed (the barrier that follows publishes them)
+    auto fills_done = []() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
+
+    // per-lane byte offsets of the MFMA operand reads inside a tile
+    uint32_t koff[KS];  // K fragment of contraction step s, key block 0 (block 1: + 32 rows)
 #pragma unroll
-        for (int i = 0; i < KLD; ++i) store_k1(buf, i);
-    };
-    auto store_v = [&](int buf) {
+    for (int sx = 0; sx < KS; ++sx) koff[sx] = (uint32_t)lq * ROWB + (uint32_t)((2 * sx + lh) ^ ksw(lq)) * 16u;
+    uint32_t voff[DB];  // V fragment of dim block b, key step 0 (step ks: + 16 ks rows; second half: + 8 rows)
+    {
+        const int t = lq & 15, r = 4 * lh + (t >> 2);
 #pragma unroll
-        for (int i = 0; i < KLD; ++i) store_v1(buf, i);
+        for (int bx = 0; bx < DB; ++bx)
+            voff[bx] = (uint32_t)r * ROWB + (uint32_t)(bx ^ vsw(r)) * 64u + (uint32_t)((lq & 16) + 4 * (t & 3)) * 2u;
+    }
+    auto read_k = [&](const uint16_t* tile, int j) {  // j = 2 s + kb
+        return *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(tile) + koff[j >> 1] + (j & 1) * 32 * ROWB);
+    };
+    auto read_v = [&](const uint16_t* tile, int j) {  // j = DB ks + b
+        typedef __attribute__((address_space(3))) ksa_short4* lds_ptr;
+        const char* pv = reinterpret_cast<const char*>(tile) + voff[j % DB] + (j / DB) * 16 * ROWB;
+        const u32x2 l2 = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(pv)));
+        const u32x2 h2 = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(pv + 8 * ROWB)));
+        u32x4 f;
+        f[0] = l2[0];
+        f[1] = l2[1];
+        f[2] = h2[0];
+        f[3] = h2[1];
+        return f;
     };
 
     // ---- walk order ----
@@ -309,13 +344,12 @@ __global__ __launch_bounds__(kThreads, (RB == 1 ? 2 : 1)) void ksa_prefill_kerne
         return z;
     };
 
-    auto scores = [&](floatx16 (&sacc)[RB][2], int buf) {  // S^T = K Q^T for the tile in Ks[buf]
+    auto scores = [&](floatx16 (&sacc)[RB][2], const uint16_t* ktile) {  // S^T = K Q^T
 #pragma unroll
         for (int s = 0; s < KS; ++s) {
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb) {
-                const u32x4 a = *reinterpret_cast<const u32x4*>(
-                    &Ks[buf][(kb * 32 + lq) * KROW + 16 * s + 8 * lh]);
+                const u32x4 a = read_k(ktile, 2 * s + kb);
 #pragma unroll
                 for (int r = 0; r < RB; ++r) {
                     if constexpr (RB == 1) {
@@ -330,20 +364,19 @@ __global__ __launch_bounds__(kThreads, (RB == 1 ? 2 : 1)) void ksa_prefill_kerne
         if constexpr (RB != 1) ksa_mfma_settle();
     };
 
-    // One pipeline step for tile `it`: its scores are in `scur`; the scores of tile it+1
-    // are produced into `snext`.  On entry LDS holds (or is being written with) K(it+1) and
-    // V(it), and the registers hold K(it+2) and V(it+1).  The barrier publishes the LDS tiles;
-    // the staging registers are written to the buffers freed by the previous step in the
-    // shadow of the score MFMAs and refilled from global memory in the shadow of the second
-    // product's, so that no wave ever sits in a block of loads or LDS stores with the matrix
-    // unit idle.
+    // One pipeline step for tile `it` (parity tag = it % 2): its scores are in `scur`; the
+    // scores of tile it+1 are produced into `snext`.  On entry the fills of K(it+1) and V(it)
+    // have landed; the barrier publishes them and frees the other two buffers, which this step
+    // refills with K(it+2) and V(it+1) while it computes.
     // `quick`: a row is visible as a whole iff it is a text row (leading prefix tiles).
-    auto step = [&](auto general_tag, int it, floatx16 (&scur)[RB][2], floatx16 (&snext)[RB][2], bool quick) {
+    auto step = [&](auto general_tag, auto parity_tag, int it, floatx16 (&scur)[RB][2],
+                    floatx16 (&snext)[RB][2], bool quick) {
         constexpr bool kGeneral = decltype(general_tag)::value;
+        constexpr int PAR = decltype(parity_tag)::value;
         const int n0 = seq(it, it) * kTileN;
-        // Past the end of the walk the pipeline keeps running on the last tile (loads) and
+        // Past the end of the walk the pipeline keeps running on the last tile (fills) and
         // on stale LDS contents (scores); those results are never used.
-        const int ik = min(it + 3, ntiles - 1), iv = min(it + 2, ntiles - 1);
+        const int ik = min(it + 2, ntiles - 1), iv = min(it + 1, ntiles - 1);
         const int nk = seq(ik, it), nv = seq(iv, it);
         const uint32_t wk = seq_word(ik, it), wv = seq_word(iv, it);
         bool row_vis[RB];
@@ -359,12 +392,12 @@ __global__ __launch_bounds__(kThreads, (RB == 1 ? 2 : 1)) void ksa_prefill_kerne
         constexpr int kQueue = 4;
         constexpr int NQK = 2 * KS;   // K fragments: contraction step s = j / 2, key block kb = j % 2
         constexpr int NPV = 4 * DB;   // V fragments: key step ks = j / DB, dim block j % DB
-        const uint16_t* ksrc = Ks[(it + 1) & 1];
-        const uint16_t* vsrc = Vs[it & 1];
-        auto kfrag = [&](int j) {
-            return *reinterpret_cast<const u32x4*>(&ksrc[((j & 1) * 32 + lq) * KROW + 16 * (j >> 1) + 8 * lh]);
-        };
-        auto vfrag = [&](int j) { return ksa_read_vt_frag<VROW>(vsrc, j / DB, j % DB, lq, lh); };
+        const uint16_t* ksrc = PAR ? Ks0 : Ks1;   // K(it+1)
+        const uint16_t* vsrc = PAR ? Vs1 : Vs0;   // V(it)
+        uint16_t* kdst = PAR ? Ks1 : Ks0;         // <- K(it+2)
+        uint16_t* vdst = PAR ? Vs0 : Vs1;         // <- V(it+1)
+        auto kfrag = [&](int j) { return read_k(ksrc, j); };
+        auto vfrag = [&](int j) { return read_v(vsrc, j); };
         u32x4 fq[kQueue];
 #pragma unroll
         for (int j = 0; j < kQueue; ++j) fq[j] = kfrag(j);
@@ -486,14 +519,11 @@ __global__ __launch_bounds__(kThreads, (RB == 1 ? 2 : 1)) void ksa_prefill_kerne
 
         // Score MFMAs of the NEXT tile with the probability pairs of THIS tile between them.
         // The fences pin the order; kLead slots run first and cover the first operand reads.
-        // The second half of the loop also carries the LDS stores of the staging registers:
-        // K(it+2) and V(it+1) go to the buffers whose last readers finished before this step's
-        // barrier (the LDS queue of a wave is idle here and saturated in the second product).
+        // The first slots also issue the fills of the two buffers freed by the barrier.
         constexpr int CPM = 16 / NQK;            // probability pairs per score MFMA
         constexpr int kLead = 3;
         constexpr int NM = NQK * RB;
-        constexpr int kStoreStep = (NM / 2) / (2 * KLD);
-        static_assert(kStoreStep >= 1, "one LDS store per MFMA slot at most");
+        static_assert(2 * KLD <= NM, "one fill per MFMA slot at most");
 #pragma unroll
         for (int vt = 0; vt < kLead; ++vt) prob_slot(vt);
         __builtin_amdgcn_sched_barrier(0);
@@ -513,11 +543,8 @@ __global__ __launch_bounds__(kThreads, (RB == 1 ? 2 : 1)) void ksa_prefill_kerne
                 const int m = j * RB + r;
 #pragma unroll
                 for (int vt = kLead + m * CPM; vt < kLead + (m + 1) * CPM; ++vt) prob_slot(vt);
-                if (m >= NM / 2 && (m - NM / 2) % kStoreStep == 0) {
-                    const int si = (m - NM / 2) / kStoreStep;
-                    if (si < KLD) store_k1(it & 1, si);
-                    else if (si < 2 * KLD) store_v1((it + 1) & 1, si - KLD);
-                }
+                if (m < KLD) fill1(kbase, kdst, kcol, nk, wk, m);
+                else if (m < 2 * KLD) fill1(vbase, vdst, vcol, nv, wv, m - KLD);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -560,7 +587,7 @@ __global__ __launch_bounds__(kThreads, (RB == 1 ? 2 : 1)) void ksa_prefill_kerne
 #pragma unroll
         for (int r = 0; r < RB; ++r) l_run[r] += l_tile[r];
 
-        // O^T += V^T P^T; the staging registers are refilled with K(it+3) and V(it+2).
+        // O^T += V^T P^T
 #pragma unroll
         for (int j = 0; j < NPV; ++j) {
 #pragma unroll
@@ -569,10 +596,9 @@ __global__ __launch_bounds__(kThreads, (RB == 1 ? 2 : 1)) void ksa_prefill_kerne
                 else Ops::mfma_a(oacc[r][j % DB], fq[j % kQueue], pf[r][j / DB]);
             }
             if (j + kQueue < NPV) fq[j % kQueue] = vfrag(j + kQueue);
-            if (j == 0) load_kv(kbase, kreg, nk, wk);
-            if (j == NPV / 4) load_kv(vbase, vreg, nv, wv);
             __builtin_amdgcn_sched_barrier(0);
         }
+        fills_done();
         if ((it & 63) == 63) {  // roll the index chunk
             seq_cur = seq_nxt;
             word_cur = word_nxt;
@@ -582,18 +608,14 @@ __global__ __launch_bounds__(kThreads, (RB == 1 ? 2 : 1)) void ksa_prefill_kerne
     };
 
     floatx16 s0[RB][2], s1[RB][2];
-    if (ntiles > 0) {  // prologue: K(0), K(1), V(0) in LDS, scores of tile 0, K(2), V(1) in registers
-        const int i1 = min(1, ntiles - 1), i2 = min(2, ntiles - 1);
-        load_kv(kbase, kreg, seq(0, 0), seq_word(0, 0));
-        load_kv(vbase, vreg, seq(0, 0), seq_word(0, 0));
-        store_k(0);
-        store_v(0);
-        load_kv(kbase, kreg, seq(i1, 0), seq_word(i1, 0));
-        load_kv(vbase, vreg, seq(i1, 0), seq_word(i1, 0));
-        store_k(1);
+    if (ntiles > 0) {  // prologue: K(0), V(0), K(1) in LDS, scores of tile 0
+        const int i1 = min(1, ntiles - 1);
+        fill(kbase, Ks0, kcol, seq(0, 0), seq_word(0, 0));
+        fill(vbase, Vs0, vcol, seq(0, 0), seq_word(0, 0));
+        fill(kbase, Ks1, kcol, seq(i1, 0), seq_word(i1, 0));
+        fills_done();
         __syncthreads();
-        load_kv(kbase, kreg, seq(i2, 0), seq_word(i2, 0));
-        scores(s0, 0);
+        scores(s0, Ks0);
     }
     auto copy_scores = [&]() {
 #pragma unroll
@@ -603,21 +625,28 @@ __global__ __launch_bounds__(kThreads, (RB == 1 ? 2 : 1)) void ksa_prefill_kerne
 #pragma unroll
                 for (int i = 0; i < 16; ++i) s0[r][kb][i] = s1[r][kb][i];
     };
+    using Even = std::integral_constant<int, 0>;
+    using Odd = std::integral_constant<int, 1>;
     int it = 0;
     for (; it + 2 <= n_a; it += 2) {
-        step(std::false_type{}, it, s0, s1, it < nquick);
-        step(std::false_type{}, it + 1, s1, s0, it + 1 < nquick);
+        step(std::false_type{}, Even{}, it, s0, s1, it < nquick);
+        step(std::false_type{}, Odd{}, it + 1, s1, s0, it + 1 < nquick);
     }
     if (it < n_a) {
-        step(std::false_type{}, it, s0, s1, it < nquick);
+        step(std::false_type{}, Even{}, it, s0, s1, it < nquick);
+        copy_scores();
+        ++it;
+    }
+    if ((it & 1) && it < ntiles) {  // phase B starts on an odd tile: one step to realign
+        step(std::true_type{}, Odd{}, it, s0, s1, false);
         copy_scores();
         ++it;
     }
     for (; it + 2 <= ntiles; it += 2) {
-        step(std::true_type{}, it, s0, s1, false);
-        step(std::true_type{}, it + 1, s1, s0, false);
+        step(std::true_type{}, Even{}, it, s0, s1, false);
+        step(std::true_type{}, Odd{}, it + 1, s1, s0, false);
     }
-    if (it < ntiles) step(std::true_type{}, it, s0, s1, false);
+    if (it < ntiles) step(std::true_type{}, Even{}, it, s0, s1, false);
 
     // ---- epilogue ----
     if constexpr (RB != 1) ksa_mfma_settle();
