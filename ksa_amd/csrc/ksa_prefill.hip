@@ -322,19 +322,9 @@ __global__ __launch_bounds__(kThreads, (RB == 1 ? 2 : 1)) void ksa_prefill_kerne
     };
 
     floatx16 oacc[RB][DB];
-    // reference maximum of the exponents (raw score units); a finite "minus huge" start
-    // value makes the first visible tile rescale the (still zero) accumulators by 0
-    float m_ref[RB];
+    float m_ref[RB];  // reference of the exponents (raw score units), see `walk` below
     float l_run[RB];  // this lane's half of the row sum
-#pragma unroll
-    for (int r = 0; r < RB; ++r) {
-        m_ref[r] = -1e30f;
-        l_run[r] = 0.f;
-#pragma unroll
-        for (int b = 0; b < DB; ++b)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) oacc[r][b][i] = 0.f;
-    }
+    bool bad = false; // optimistic walk: some exponent left the safe range
     const float c2 = p.scale_log2;
 
     auto zero16 = []() {
@@ -344,7 +334,7 @@ __global__ __launch_bounds__(kThreads, (RB == 1 ? 2 : 1)) void ksa_prefill_kerne
         return z;
     };
 
-    auto scores = [&](floatx16 (&sacc)[RB][2], const uint16_t* ktile) {  // S^T = K Q^T
+    auto scores = [&](floatx16 (&sacc)[RB][2], const uint16_t* ktile) __attribute__((always_inline)) {  // S^T = K Q^T
 #pragma unroll
         for (int s = 0; s < KS; ++s) {
 #pragma unroll
@@ -369,8 +359,9 @@ __global__ __launch_bounds__(kThreads, (RB == 1 ? 2 : 1)) void ksa_prefill_kerne
     // have landed; the barrier publishes them and frees the other two buffers, which this step
     // refills with K(it+2) and V(it+1) while it computes.
     // `quick`: a row is visible as a whole iff it is a text row (leading prefix tiles).
-    auto step = [&](auto general_tag, auto parity_tag, int it, floatx16 (&scur)[RB][2],
-                    floatx16 (&snext)[RB][2], bool quick) {
+    auto step = [&](auto safe_tag, auto general_tag, auto parity_tag, int it, floatx16 (&scur)[RB][2],
+                    floatx16 (&snext)[RB][2], bool quick) __attribute__((always_inline)) {
+        constexpr bool kSafe = decltype(safe_tag)::value;
         constexpr bool kGeneral = decltype(general_tag)::value;
         constexpr int PAR = decltype(parity_tag)::value;
         const int n0 = seq(it, it) * kTileN;
@@ -426,10 +417,10 @@ __global__ __launch_bounds__(kThreads, (RB == 1 ? 2 : 1)) void ksa_prefill_kerne
             }
         }
 
-        // Probabilities relative to the current reference.  The row maximum is computed
-        // only where it is needed: always on the masked tiles of phase B; on phase A tiles
-        // only after the fact, when a row has no reference yet or its tile sum shows that the
-        // exponents outgrew the reference (then the tile's probabilities are redone).
+        // Probabilities relative to the current reference.  The row maximum is computed only
+        // where it is needed: on the masked tiles of phase B and in the safe walk.  The
+        // optimistic walk keeps the reference it has on phase A tiles and only watches the
+        // tile sums.
         float l_tile[RB];
         u32x4 pf[RB][4];
         float mc[RB];
@@ -511,7 +502,7 @@ __global__ __launch_bounds__(kThreads, (RB == 1 ? 2 : 1)) void ksa_prefill_kerne
                 }
             }
         };
-        if constexpr (kGeneral) {
+        if constexpr (kGeneral || kSafe) {
             rebase();
 #pragma unroll
             for (int r = 0; r < RB; ++r) mc[r] = row_vis[r] ? m_ref[r] * c2 : INFINITY;
@@ -548,41 +539,10 @@ __global__ __launch_bounds__(kThreads, (RB == 1 ? 2 : 1)) void ksa_prefill_kerne
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
-        if constexpr (!kGeneral) {
-            // 2^24: some exponent exceeded the reference by more than ~19; also true for the
-            // first visible tile of a row (reference still "minus huge" -> infinite sum).
-            // The scores were given up register by register as the pairs consumed them, so
-            // this rare path first recomputes them, with K fragments straight from global
-            // memory (the tile's LDS buffer may already be in the hands of a faster wave).
-            bool redo = false;
+        if constexpr (!kGeneral && !kSafe) {
+            // 2^24: some exponent exceeded the reference by more than ~19
 #pragma unroll
-            for (int r = 0; r < RB; ++r) redo = redo || l_tile[r] > 16777216.f;
-#ifdef KSA_X_NOREDO
-            if (false) {
-#else
-            if (__any(redo)) {
-#endif
-#pragma unroll
-                for (int sx = 0; sx < KS; ++sx)
-#pragma unroll
-                    for (int kb = 0; kb < 2; ++kb) {
-                        const uint32_t row = src_row(n0 + kb * 32 + lq);
-                        const u32x4 a = *reinterpret_cast<const u32x4*>(
-                            kbase + (size_t)row * rb + (uint32_t)(16 * sx + 8 * lh) * 2u);
-#pragma unroll
-                        for (int r = 0; r < RB; ++r) {
-                            if constexpr (RB == 1) {
-                                scur[r][kb] = Ops::mfma(a, qf[r][sx], sx == 0 ? zero16() : scur[r][kb]);
-                            } else {
-                                if (sx == 0) scur[r][kb] = Ops::mfma_v0(a, qf[r][sx]);
-                                else Ops::mfma_v(scur[r][kb], a, qf[r][sx]);
-                            }
-                        }
-                    }
-                if constexpr (RB != 1) ksa_mfma_settle();
-                rebase();
-                probabilities();
-            }
+            for (int r = 0; r < RB; ++r) bad = bad || l_tile[r] > 16777216.f;
         }
 #pragma unroll
         for (int r = 0; r < RB; ++r) l_run[r] += l_tile[r];
@@ -607,17 +567,15 @@ __global__ __launch_bounds__(kThreads, (RB == 1 ? 2 : 1)) void ksa_prefill_kerne
         }
     };
 
+    // One complete walk over the tile list.  The optimistic walk (kSafe = false) takes each
+    // row's reference from the unmasked scores of the first tile and never moves it on phase A
+    // tiles; it reports when that went wrong -- an exponent far above the reference (tile sum
+    // above 2^24) or a row sum so small that the reference was far too high -- and the
+    // workgroup then repeats the walk in the safe form, which moves the reference before the
+    // probabilities of every tile (the textbook online soft-max, still with the lazy
+    // threshold).  Random-like scores never need the second walk.
     floatx16 s0[RB][2], s1[RB][2];
-    if (ntiles > 0) {  // prologue: K(0), V(0), K(1) in LDS, scores of tile 0
-        const int i1 = min(1, ntiles - 1);
-        fill(kbase, Ks0, kcol, seq(0, 0), seq_word(0, 0));
-        fill(vbase, Vs0, vcol, seq(0, 0), seq_word(0, 0));
-        fill(kbase, Ks1, kcol, seq(i1, 0), seq_word(i1, 0));
-        fills_done();
-        __syncthreads();
-        scores(s0, Ks0);
-    }
-    auto copy_scores = [&]() {
+    auto copy_scores = [&]() __attribute__((always_inline)) {
 #pragma unroll
         for (int r = 0; r < RB; ++r)
 #pragma unroll
@@ -627,26 +585,73 @@ __global__ __launch_bounds__(kThreads, (RB == 1 ? 2 : 1)) void ksa_prefill_kerne
     };
     using Even = std::integral_constant<int, 0>;
     using Odd = std::integral_constant<int, 1>;
-    int it = 0;
-    for (; it + 2 <= n_a; it += 2) {
-        step(std::false_type{}, Even{}, it, s0, s1, it < nquick);
-        step(std::false_type{}, Odd{}, it + 1, s1, s0, it + 1 < nquick);
+    auto walk = [&](auto safe_tag) __attribute__((always_inline)) {
+        constexpr bool kSafe = decltype(safe_tag)::value;
+        using A = std::false_type;
+        using B = std::true_type;
+        seq_cur = seq_chunk(0);
+        seq_nxt = seq_chunk(64);
+        word_cur = kRegular ? tile_word(seq_cur) : 0u;
+        word_nxt = kRegular ? tile_word(seq_nxt) : 0u;
+#pragma unroll
+        for (int r = 0; r < RB; ++r) {
+            m_ref[r] = -1e30f;  // finite: the first rescale multiplies the zero accumulators by 0
+            l_run[r] = 0.f;
+#pragma unroll
+            for (int b = 0; b < DB; ++b)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) oacc[r][b][i] = 0.f;
+        }
+        if (ntiles > 0) {  // prologue: K(0), V(0), K(1) in LDS, scores of tile 0
+            const int i1 = min(1, ntiles - 1);
+            fill(kbase, Ks0, kcol, seq(0, 0), seq_word(0, 0));
+            fill(vbase, Vs0, vcol, seq(0, 0), seq_word(0, 0));
+            fill(kbase, Ks1, kcol, seq(i1, 0), seq_word(i1, 0));
+            fills_done();
+            __syncthreads();
+            scores(s0, Ks0);
+            if constexpr (!kSafe) {
+#pragma unroll
+                for (int r = 0; r < RB; ++r) {
+                    float mloc = fmaxf(s0[r][0][0], s0[r][1][0]);
+#pragma unroll
+                    for (int i = 1; i < 16; ++i) mloc = fmaxf(mloc, fmaxf(s0[r][0][i], s0[r][1][i]));
+                    m_ref[r] = ksa_pair_max(mloc);
+                }
+            }
+        }
+        int it = 0;
+        for (; it + 2 <= n_a; it += 2) {
+            step(safe_tag, A{}, Even{}, it, s0, s1, it < nquick);
+            step(safe_tag, A{}, Odd{}, it + 1, s1, s0, it + 1 < nquick);
+        }
+        if (it < n_a) {
+            step(safe_tag, A{}, Even{}, it, s0, s1, it < nquick);
+            copy_scores();
+            ++it;
+        }
+        if ((it & 1) && it < ntiles) {  // phase B starts on an odd tile: one step to realign
+            step(safe_tag, B{}, Odd{}, it, s0, s1, false);
+            copy_scores();
+            ++it;
+        }
+        for (; it + 2 <= ntiles; it += 2) {
+            step(safe_tag, B{}, Even{}, it, s0, s1, false);
+            step(safe_tag, B{}, Odd{}, it + 1, s1, s0, false);
+        }
+        if (it < ntiles) step(safe_tag, B{}, Even{}, it, s0, s1, false);
+    };
+
+    walk(std::false_type{});
+    {
+#pragma unroll
+        for (int r = 0; r < RB; ++r) {
+            const float l_tot = ksa_pair_sum(l_run[r]);
+            // every row sees at least itself: a vanishing sum means a reference far too high
+            bad = bad || !(l_tot > 5.4e-20f);
+        }
+        if (__syncthreads_or(bad)) walk(std::true_type{});
     }
-    if (it < n_a) {
-        step(std::false_type{}, Even{}, it, s0, s1, it < nquick);
-        copy_scores();
-        ++it;
-    }
-    if ((it & 1) && it < ntiles) {  // phase B starts on an odd tile: one step to realign
-        step(std::true_type{}, Odd{}, it, s0, s1, false);
-        copy_scores();
-        ++it;
-    }
-    for (; it + 2 <= ntiles; it += 2) {
-        step(std::true_type{}, Even{}, it, s0, s1, false);
-        step(std::true_type{}, Odd{}, it + 1, s1, s0, false);
-    }
-    if (it < ntiles) step(std::true_type{}, Even{}, it, s0, s1, false);
 
     // ---- epilogue ----
     if constexpr (RB != 1) ksa_mfma_settle();
