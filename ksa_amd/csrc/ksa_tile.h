@@ -44,17 +44,19 @@ struct KsaOps<KsaBf16> {
     // files: accumulators of the second product (`acc`) and the resident B operand of the
     // first (`b_acc`) live in AGPRs, scores and LDS-fed operands in VGPRs.  The compiler does
     // not see an MFMA in these statements, so the caller keeps MFMA results away from vector
-    // instructions for the required wait states (ksa_mfma_settle).
+    // instructions for the required wait states (ksa_mfma_settle), and each statement carries
+    // the one wait state the hardware needs between a vector instruction and an MFMA (without
+    // it the first MFMA after vector work computed garbage on gfx950).
     static __device__ __forceinline__ floatx16 mfma_v0(u32x4 a, u32x4 b_acc) {
         floatx16 d;
-        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "a"(b_acc));
+        asm volatile("s_nop 0\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "a"(b_acc));
         return d;
     }
     static __device__ __forceinline__ void mfma_v(floatx16& c, u32x4 a, u32x4 b_acc) {
-        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b_acc));
+        asm volatile("s_nop 0\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b_acc));
     }
     static __device__ __forceinline__ void mfma_a(floatx16& acc, u32x4 a, u32x4 b) {
-        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+        asm volatile("s_nop 0\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
     }
     static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
         bf16x2 v;
@@ -79,14 +81,14 @@ struct KsaOps<KsaF16> {
     }
     static __device__ __forceinline__ floatx16 mfma_v0(u32x4 a, u32x4 b_acc) {
         floatx16 d;
-        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "a"(b_acc));
+        asm volatile("s_nop 0\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "a"(b_acc));
         return d;
     }
     static __device__ __forceinline__ void mfma_v(floatx16& c, u32x4 a, u32x4 b_acc) {
-        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b_acc));
+        asm volatile("s_nop 0\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b_acc));
     }
     static __device__ __forceinline__ void mfma_a(floatx16& acc, u32x4 a, u32x4 b) {
-        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+        asm volatile("s_nop 0\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
     }
     static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
         f16x2 v;

@@ -77,6 +77,18 @@ def test_index_cfg2_known_answer():
     assert int((idx[0] + idx[2]).max()) == 139
 
 
+@pytest.fixture(params=[None, "64"], ids=["rows32", "rows64"])
+def wave_rows(request, monkeypatch):
+    """Both workgroup shapes of the prefill kernel: 32 query rows per wave (default) and the
+    two-heads-per-workgroup variant with 64 rows per wave (KSA_PREFILL_ROWS_PER_WAVE=64, read
+    by the library on every call; it applies to D = 128 with an even group size)."""
+    if request.param is None:
+        monkeypatch.delenv("KSA_PREFILL_ROWS_PER_WAVE", raising=False)
+    else:
+        monkeypatch.setenv("KSA_PREFILL_ROWS_PER_WAVE", request.param)
+    return request.param
+
+
 def _run_prefill(q, k, v, C, S, W, summary_pos, skip_old=False, **kw):
     import ksa_amd
     dev = torch.device("cuda")
@@ -97,7 +109,7 @@ def _compare(got, want, what):
 
 
 @pytest.mark.parametrize("W", [3, 4])
-def test_prefill_cfg0_full_compare(W):
+def test_prefill_cfg0_full_compare(W, wave_rows):
     """cfg 0: 32 chunks x (128+8), 16 q heads / 8 kv heads, D=128, every output row."""
     Sq, Hq, Hkv, D, C, S = 4352, 16, 8, 128, 128, 8
     q, k, v = make_qkv(Sq, Hq, Hkv, D, seed=0)
@@ -135,7 +147,7 @@ def test_prefill_unscaled_logits(scaled):
     (130, 2, 2, 128, 128, 8, 0, "prefix", False),          # shorter than one block + tail
     (64, 2, 1, 128, 128, 8, 4, "prefix", False),           # no summaries at all
 ])
-def test_prefill_variants(case):
+def test_prefill_variants(case, wave_rows):
     Sq, Hq, Hkv, D, C, S, W, mode, skip_old = case
     q, k, v = make_qkv(Sq, Hq, Hkv, D, seed=2, scaled=False)
     sp = O.summary_positions(Sq, C, S)
@@ -189,7 +201,7 @@ def test_prefill_visibility_probe():
     assert np.abs(got[:, 1] - want).max() <= 4e-3
 
 
-def test_prefill_cfg1_sampled_rows():
+def test_prefill_cfg1_sampled_rows(wave_rows):
     """cfg 1 (32k text tokens, 32/8 heads): rows of the first and last two chunks, offsets
     {0, C-1, C, B-1} of 64 random chunks and 1024 random rows against the oracle."""
     Sq, Hq, Hkv, D, C, S, W = 34816, 32, 8, 128, 128, 8, 4
@@ -208,7 +220,7 @@ def test_prefill_cfg1_sampled_rows():
     assert np.abs(lse[:, rows] - wlse).max() <= 2e-3
 
 
-def test_prefill_batch_and_fp16():
+def test_prefill_batch_and_fp16(wave_rows):
     Sq, Hq, Hkv, D, C, S, W = 680, 4, 2, 128, 128, 8, 1
     import ksa_amd
     dev = torch.device("cuda")
@@ -245,7 +257,7 @@ def test_prefill_rejects_bad_inputs():
         ksa_amd.summary_attn_func(qg, q, q, 128, 8, 1)
 
 
-def test_prefill_growing_scores_rebase():
+def test_prefill_growing_scores_rebase(wave_rows):
     """Scores that grow strongly along the key axis (later tiles exceed every earlier row
     maximum by far) force the soft-max reference to move many times, including on tiles that
     take the no-maximum fast path; a stale reference would overflow or lose the early keys."""
@@ -266,7 +278,7 @@ def test_prefill_growing_scores_rebase():
     assert np.abs(lse[:, rows] - wlse).max() <= 0.1
 
 
-def test_prefill_decreasing_scores():
+def test_prefill_decreasing_scores(wave_rows):
     """The opposite order: the first tiles hold the largest logits, everything later is far
     below the reference (probabilities underflow gracefully, nothing is rescaled)."""
     Sq, Hq, Hkv, D, C, S, W = 48 * 136, 4, 2, 128, 128, 8, 3
@@ -280,3 +292,23 @@ def test_prefill_decreasing_scores():
     want, _ = c_oracle.attention_rows(to_np(q), to_np(k), to_np(v), C, S, W, summary_pos=sp, rows=rows)
     err = np.abs(got[rows] - want).max()
     assert err <= ATOL * max(1.0, np.abs(want).max()), err
+
+
+def test_prefill_reference_far_too_high(wave_rows):
+    """Summary keys with a huge norm: text rows see them, the summary rows of the same query
+    tile do not, so a soft-max reference taken from the unmasked first tile is hundreds of
+    octaves above everything a summary row sees and all its probabilities underflow.  The
+    kernel has to notice (vanishing row sum) and redo the tile walk with exact references."""
+    Sq, Hq, Hkv, D, C, S, W = 24 * 136, 4, 2, 128, 128, 8, 2
+    q, k, v = make_qkv(Sq, Hq, Hkv, D, seed=9, scaled=False)
+    sp = O.summary_positions(Sq, C, S)
+    boost = torch.ones(Sq)
+    boost[torch.as_tensor(sp)] = 40.0
+    k = (k.float() * boost[:, None, None]).to(torch.bfloat16)
+    got, lse = _run_prefill(q, k, v, C, S, W, sp)
+    rows = np.r_[0:Sq:7].astype(np.int32)
+    want, wlse = c_oracle.attention_rows(to_np(q), to_np(k), to_np(v), C, S, W, summary_pos=sp, rows=rows)
+    assert np.isfinite(got).all()
+    err = np.abs(got[rows] - want).max()
+    assert err <= ATOL * max(1.0, np.abs(want).max()), err
+    assert np.abs(lse[:, rows] - wlse).max() <= 0.1 + 1e-3 * np.abs(wlse).max()
