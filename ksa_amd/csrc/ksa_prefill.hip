@@ -57,10 +57,9 @@ struct PrefillParams {
     KsaMask mk;
     float scale;
     float scale_log2;
-    int rows_per_wave;  // 64: two row blocks per wave where the shape allows (experimental)
+    int shape;  // 0: default; 32: one head per workgroup; 64: two heads, 64 query rows per wave
 };
 
-constexpr int kThreads = 256;
 constexpr int kTileM = 128;
 constexpr int kTileN = 64;
 
@@ -106,8 +105,21 @@ __device__ __forceinline__ RowVis ksa_row_vis(const KsaMask& mk, int q) {
 // CU with up to 512 registers per lane; every K and V fragment read from LDS then feeds two
 // MFMAs, which halves the LDS traffic per MFMA (at one fragment per MFMA the four SIMDs ask
 // for more than the LDS delivers).
-template <typename T, int D, bool kRegular, int RB>
-__global__ __launch_bounds__(kThreads, (RB == 1 ? 2 : 1)) void ksa_prefill_kernel(const PrefillParams p) {
+//
+// HW: query heads (of one kv group) per workgroup.  The workgroup has 4 HW / RB waves; with
+// HW = 2, RB = 1 (8 waves, two per SIMD) one K/V tile in LDS serves twice the MFMA work, which
+// halves the fill traffic into LDS per MFMA.
+template <int RB, int HW>
+struct PrefillShape {
+    static constexpr int kWaves = 4 * HW / RB;
+    static constexpr int kThreads = 64 * kWaves;
+    static constexpr int kWavesPerSimd = kWaves * (RB == 1 && HW == 1 ? 2 : 1) / 4;  // 2, 1 or 2
+};
+
+template <typename T, int D, bool kRegular, int RB, int HW>
+__global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)) void ksa_prefill_kernel(
+    const PrefillParams p) {
+    constexpr int kThreads = PrefillShape<RB, HW>::kThreads;
     using Ops = KsaOps<T>;
     constexpr int KS = D / 16;       // contraction steps of K Q^T
     constexpr int DB = D / 32;       // 32-row blocks of O^T
@@ -143,11 +155,12 @@ __global__ __launch_bounds__(kThreads, (RB == 1 ? 2 : 1)) void ksa_prefill_kerne
     const int id = blockIdx.x;
     const int kvh = id % p.Hkv;
     const int rest = id / p.Hkv;
-    const int gper = p.g / RB;
+    constexpr int kWavesPerHead = 4 / RB;
+    const int gper = p.g / HW;
     const int gi = rest % gper;
     const int mt = p.M - 1 - rest / gper;
-    const int head = kvh * p.g + (RB == 1 ? gi : 2 * gi + (wave >> 1));
-    const int row0 = mt * kTileM + (RB == 1 ? wave * 32 : (wave & 1) * 64);
+    const int head = kvh * p.g + HW * gi + wave / kWavesPerHead;
+    const int row0 = mt * kTileM + (wave % kWavesPerHead) * 32 * RB;
     const KsaMask mk = p.mk;
     const bool prefix_mode = mk.P > 0;
     const bool phys = p.phys_prefix != 0;
@@ -677,30 +690,31 @@ __global__ __launch_bounds__(kThreads, (RB == 1 ? 2 : 1)) void ksa_prefill_kerne
     }
 }
 
-template <typename T, int D>
-int launch(const PrefillParams& p, int batch, hipStream_t stream) {
+template <typename T, int D, int RB, int HW>
+int launch_shape(const PrefillParams& p, int batch, hipStream_t stream) {
+    constexpr int kThreads = PrefillShape<RB, HW>::kThreads;
     constexpr int RSTEP = kThreads / (D / 8);
     const KsaMask& mk = p.mk;
     const bool prefix_ok = mk.P == 0 || p.phys_prefix || (RSTEP % mk.S == 0 && mk.P % kTileN == 0);
     const bool regular = prefix_ok && mk.Sk % kTileN == 0;
-    // two heads per workgroup need an even group size; the wider kernel is built for D = 128
-    const bool pair = D == 128 && p.g % 2 == 0 && p.rows_per_wave == 64;
-    if (pair) {
-        dim3 grid(p.M * (p.Hq / 2), batch);
-        if constexpr (D == 128) {
-            if (regular)
-                hipLaunchKernelGGL((ksa_prefill_kernel<T, D, true, 2>), grid, dim3(kThreads), 0, stream, p);
-            else
-                hipLaunchKernelGGL((ksa_prefill_kernel<T, D, false, 2>), grid, dim3(kThreads), 0, stream, p);
-        }
-    } else {
-        dim3 grid(p.M * p.Hq, batch);
-        if (regular)
-            hipLaunchKernelGGL((ksa_prefill_kernel<T, D, true, 1>), grid, dim3(kThreads), 0, stream, p);
-        else
-            hipLaunchKernelGGL((ksa_prefill_kernel<T, D, false, 1>), grid, dim3(kThreads), 0, stream, p);
-    }
+    dim3 grid(p.M * (p.Hq / HW), batch);
+    if (regular)
+        hipLaunchKernelGGL((ksa_prefill_kernel<T, D, true, RB, HW>), grid, dim3(kThreads), 0, stream, p);
+    else
+        hipLaunchKernelGGL((ksa_prefill_kernel<T, D, false, RB, HW>), grid, dim3(kThreads), 0, stream, p);
     return ksa_check_launch();
+}
+
+template <typename T, int D>
+int launch(const PrefillParams& p, int batch, hipStream_t stream) {
+    // workgroup shapes with two heads need an even group size and are built for D = 128
+    if constexpr (D == 128) {
+        if (p.g % 2 == 0) {
+            if (p.shape == 64) return launch_shape<T, D, 2, 2>(p, batch, stream);
+            if (p.shape != 32) return launch_shape<T, D, 1, 2>(p, batch, stream);
+        }
+    }
+    return launch_shape<T, D, 1, 1>(p, batch, stream);
 }
 
 bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; }
@@ -761,10 +775,11 @@ extern "C" int ksa_prefill_fwd(const void* q, const void* k, const void* v, void
     p.mk = KsaMask{C, S, W, P, skip_old ? 1 : 0, Sq, Sk};
     p.scale = scale;
     p.scale_log2 = scale * 1.4426950408889634f;
-    // KSA_PREFILL_ROWS_PER_WAVE=64 selects the two-head workgroup (64 query rows per wave, one
-    // wave per SIMD) where the shape allows; it is correct but not yet faster
+    // Workgroup shape (D = 128, even group size; anything else uses one head per workgroup):
+    // default two heads on 8 waves; KSA_PREFILL_ROWS_PER_WAVE=32 one head on 4 waves;
+    // =64 two heads on 4 waves with 64 query rows per wave (one wave per SIMD).
     const char* rpw = getenv("KSA_PREFILL_ROWS_PER_WAVE");
-    p.rows_per_wave = rpw ? atoi(rpw) : 0;
+    p.shape = rpw ? atoi(rpw) : 0;
 
     hipStream_t st = (hipStream_t)stream;
     if (dtype == KSA_DTYPE_BF16) {

@@ -77,11 +77,11 @@ def test_index_cfg2_known_answer():
     assert int((idx[0] + idx[2]).max()) == 139
 
 
-@pytest.fixture(params=[None, "64"], ids=["rows32", "rows64"])
+@pytest.fixture(params=[None, "32", "64"], ids=["default", "rows32", "rows64"])
 def wave_rows(request, monkeypatch):
-    """Both workgroup shapes of the prefill kernel: 32 query rows per wave (default) and the
-    two-heads-per-workgroup variant with 64 rows per wave (KSA_PREFILL_ROWS_PER_WAVE=64, read
-    by the library on every call; it applies to D = 128 with an even group size)."""
+    """The workgroup shapes of the prefill kernel (D = 128, even group size): two heads on 8
+    waves (default), one head on 4 waves (KSA_PREFILL_ROWS_PER_WAVE=32) and two heads on 4
+    waves with 64 query rows per wave (=64).  The library reads the variable on every call."""
     if request.param is None:
         monkeypatch.delenv("KSA_PREFILL_ROWS_PER_WAVE", raising=False)
     else:
