@@ -252,7 +252,10 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
         typedef __attribute__((address_space(1))) void* gptr;
         typedef __attribute__((address_space(3))) void* lptr;
         char* dst = reinterpret_cast<char*>(tile) + (RSTEP * i + wave_u * (64 / CPR)) * ROWB;
-        __builtin_amdgcn_global_load_lds((gptr)(base + (ub + us * i) + vo[i] + col), (lptr)dst, 16, 0, 0);
+        // uniform 64-bit base + one 32-bit lane offset: the scalar-base addressing form
+        const char* ubase = base + (ub + us * i);
+        const uint32_t loff = vo[i] + col;
+        __builtin_amdgcn_global_load_lds((gptr)(ubase + loff), (lptr)dst, 16, 0, 0);
     };
     auto fill = [&](const char* base, uint16_t* tile, uint32_t col, int n, uint32_t word) {
 #pragma unroll
