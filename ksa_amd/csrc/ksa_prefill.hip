@@ -156,6 +156,7 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
     const int kvh = id % p.Hkv;
     const int rest = id / p.Hkv;
     constexpr int kWavesPerHead = 4 / RB;
+
     const int gper = p.g / HW;
     const int gi = rest % gper;
     const int mt = p.M - 1 - rest / gper;
@@ -249,13 +250,23 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
         } else {
             tile_src(n * kTileN, ub, us, vo);
         }
-        typedef __attribute__((address_space(1))) void* gptr;
-        typedef __attribute__((address_space(3))) void* lptr;
+        typedef __attribute__((address_space(3))) char* lptr;
         char* dst = reinterpret_cast<char*>(tile) + (RSTEP * i + wave_u * (64 / CPR)) * ROWB;
-        // uniform 64-bit base + one 32-bit lane offset: the scalar-base addressing form
-        const char* ubase = base + (ub + us * i);
+        // Uniform 64-bit base + one 32-bit lane offset (the scalar-base addressing form); M0
+        // carries the LDS address of the wave's 1 KB piece, lane l lands at + 16 l.  Written as
+        // assembly so that the compiler does not track the fill: it would otherwise make LDS
+        // reads wait for fills it cannot tell apart; which fills must have landed before a
+        // barrier is decided by fills_done.
+        const uint64_t ubase = reinterpret_cast<uint64_t>(base + (ub + us * i));
         const uint32_t loff = vo[i] + col;
-        __builtin_amdgcn_global_load_lds((gptr)(ubase + loff), (lptr)dst, 16, 0, 0);
+        const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr)dst;
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"  // M0 is reserved; nothing else in this kernel uses it
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                     :
+                     : "s"(lds_addr), "v"(loff), "s"(ubase)
+                     : "memory", "m0");
+#pragma clang diagnostic pop
     };
     auto fill = [&](const char* base, uint16_t* tile, uint32_t col, int n, uint32_t word) {
 #pragma unroll
@@ -263,6 +274,9 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
     };
     // all of this wave's fills have landed (the barrier that follows publishes them)
     auto fills_done = []() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
+    // Workgroup barrier of the tile loop: a plain s_barrier (the fills that have to be visible
+    // are awaited explicitly by fills_done; LDS reads are complete once their data was used).
+    auto wg_barrier = []() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
 
     // per-lane byte offsets of the MFMA operand reads inside a tile
     uint32_t koff[KS];  // K fragment of contraction step s, key block 0 (block 1: + 32 rows)
@@ -383,13 +397,14 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
         const int n0 = seq(it, it) * kTileN;
         // Past the end of the walk the pipeline keeps running on the last tile (fills) and
         // on stale LDS contents (scores); those results are never used.
+        // fills: K(it+2) in the score stage, V(it+1) in the second-product stage
         const int ik = min(it + 2, ntiles - 1), iv = min(it + 1, ntiles - 1);
         const int nk = seq(ik, it), nv = seq(iv, it);
         const uint32_t wk = seq_word(ik, it), wv = seq_word(iv, it);
         bool row_vis[RB];
 #pragma unroll
         for (int r = 0; r < RB; ++r) row_vis[r] = quick ? rv[r].b_text : true;
-        __syncthreads();
+        wg_barrier();
 
         // MFMA operands that come from LDS travel through a rolling queue of kQueue fragments:
         // the read for operand j + kQueue is issued right behind the MFMAs of operand j, through
@@ -530,7 +545,7 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
         constexpr int CPM = 16 / NQK;            // probability pairs per score MFMA
         constexpr int kLead = 3;
         constexpr int NM = NQK * RB;
-        static_assert(2 * KLD <= NM, "one fill per MFMA slot at most");
+        static_assert(KLD <= NM && KLD <= NPV, "one fill per MFMA slot at most");
 #pragma unroll
         for (int vt = 0; vt < kLead; ++vt) prob_slot(vt);
         __builtin_amdgcn_sched_barrier(0);
@@ -551,7 +566,6 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
 #pragma unroll
                 for (int vt = kLead + m * CPM; vt < kLead + (m + 1) * CPM; ++vt) prob_slot(vt);
                 if (m < KLD) fill1(kbase, kdst, kcol, nk, wk, m);
-                else if (m < 2 * KLD) fill1(vbase, vdst, vcol, nv, wv, m - KLD);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -572,6 +586,7 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
                 else Ops::mfma_a(oacc[r][j % DB], fq[j % kQueue], pf[r][j / DB]);
             }
             if (j + kQueue < NPV) fq[j % kQueue] = vfrag(j + kQueue);
+            if (j < KLD) fill1(vbase, vdst, vcol, nv, wv, j);
             __builtin_amdgcn_sched_barrier(0);
         }
         fills_done();
