@@ -136,8 +136,8 @@ def main():
                          "used to scale the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py measures one GPU: this build has no multi-GPU path (see DESIGN.md, "
-              "'How the paths would shard'); run with --gpus 1", file=sys.stderr)
+        print("bench.py measures one GPU: this build has no multi-GPU path (both kernels shard "
+              "by head / sequence with no communication); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
 
     import torch

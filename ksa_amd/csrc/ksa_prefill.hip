@@ -9,22 +9,31 @@
 // the scale folded in, probabilities rounded to 16 bit before the second product,
 // fp32 output accumulator, one reciprocal per row at the end.
 //
-// One workgroup (4 waves) owns a 128-row query tile of one query head; wave w owns
-// rows 32w .. 32w+31.  It walks the tile's non-empty key tiles (64 keys each) taken
-// from the block index, staging K and V row-major in LDS (two buffers each); V is
-// transposed on the way out of LDS by ds_read_b64_tr_b16 (operand layouts: ksa_tile.h).
-// The summary prefix of the key axis is read in place from the in-line summary rows
-// (or, with `phys_prefix`, from the first P rows of K/V), never concatenated.
+// A workgroup owns a 128-row query tile of one or two query heads of a kv group (shapes:
+// `PrefillShape`); a wave owns 32 (or 64) of those rows for one head.  It walks the tile's
+// non-empty key tiles (64 keys each) taken from the block index.  K and V tiles go from
+// global memory straight into LDS (global_load_lds, two buffers each, row-major with the
+// 16-byte chunks of every row XOR-permuted against bank conflicts); V is transposed on the
+// way out of LDS by ds_read_b64_tr_b16 (operand layouts: ksa_tile.h).  The summary prefix of
+// the key axis is read in place from the in-line summary rows (or, with `phys_prefix`, from
+// the first P rows of K/V), never concatenated.
 //
-// The loop is software-pipelined: the score MFMAs of tile i+1 are issued before the
-// soft-max of tile i so that matrix and vector work of one wave overlap; K therefore
-// runs one tile ahead of V through LDS.
+// The loop is software-pipelined: the score MFMAs of tile i+1 are interleaved with the
+// soft-max of tile i, one MFMA and one pair of probabilities per time slot, so that matrix
+// and vector work of one wave overlap; K therefore runs one tile ahead of V through LDS.
+// All MFMA operands that come from LDS pass through a small rolling queue of fragments that
+// is refilled right behind each MFMA.
 //
 // Masking.  The walk has two phases that are uniform for the workgroup.  Phase A holds
 // the tiles that need no per-element mask: the leading partial tiles below every text
 // row's old-summary bound (there a row is visible as a whole iff it is a text row) and
 // the full tiles.  Phase B holds the remaining partial tiles, masked per element from a
 // 64-bit visibility word per query row.
+//
+// Soft-max reference.  The first walk is optimistic: a row's reference exponent comes from
+// the unmasked scores of the first tile and is not moved on phase A tiles (no row maximum
+// is computed there); the walk only records whether an exponent left the safe range.  If
+// that ever happens the workgroup repeats the walk with the textbook online soft-max.
 #include <hip/hip_runtime.h>
 #include <math.h>
 #include <stdlib.h>
@@ -113,7 +122,6 @@ template <int RB, int HW>
 struct PrefillShape {
     static constexpr int kWaves = 4 * HW / RB;
     static constexpr int kThreads = 64 * kWaves;
-    static constexpr int kWavesPerSimd = kWaves * (RB == 1 && HW == 1 ? 2 : 1) / 4;  // 2, 1 or 2
 };
 
 template <typename T, int D, bool kRegular, int RB, int HW>
