@@ -146,6 +146,8 @@ def test_prefill_unscaled_logits(scaled):
     (1360, 4, 2, 128, 128, 8, 2, "physical", False),       # k/v already carry the prefix
     (130, 2, 2, 128, 128, 8, 0, "prefix", False),          # shorter than one block + tail
     (64, 2, 1, 128, 128, 8, 4, "prefix", False),           # no summaries at all
+    (1500, 6, 2, 128, 128, 8, 2, "prefix", False),         # odd group size (g = 3)
+    (1500, 12, 2, 128, 128, 8, 3, "prefix", False),        # g = 6: three head pairs per kv head
 ])
 def test_prefill_variants(case, wave_rows):
     Sq, Hq, Hkv, D, C, S, W, mode, skip_old = case
