@@ -31,9 +31,9 @@
 // 64-bit visibility word per query row.
 //
 // Soft-max reference.  The first walk is optimistic: a row's reference exponent comes from
-// the unmasked scores of the first tile and is not moved on phase A tiles (no row maximum
-// is computed there); the walk only records whether an exponent left the safe range.  If
-// that ever happens the workgroup repeats the walk with the textbook online soft-max.
+// the unmasked scores of the first tile and is never moved (no row maximum is computed);
+// the walk only records whether an exponent left the safe range.  If that ever happens
+// the workgroup repeats the walk with the textbook online soft-max.
 #include <hip/hip_runtime.h>
 #include <math.h>
 #include <stdlib.h>
@@ -457,9 +457,8 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
         }
 
         // Probabilities relative to the current reference.  The row maximum is computed only
-        // where it is needed: on the masked tiles of phase B and in the safe walk.  The
-        // optimistic walk keeps the reference it has on phase A tiles and only watches the
-        // tile sums.
+        // in the safe walk; the optimistic walk keeps the reference it has and only watches
+        // the tile sums.
         float l_tile[RB];
         u32x4 pf[RB][4];
         float mc[RB];
@@ -541,7 +540,7 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
                 }
             }
         };
-        if constexpr (kGeneral || kSafe) {
+        if constexpr (kSafe) {
             rebase();
 #pragma unroll
             for (int r = 0; r < RB; ++r) mc[r] = row_vis[r] ? m_ref[r] * c2 : INFINITY;
@@ -577,7 +576,7 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
-        if constexpr (!kGeneral && !kSafe) {
+        if constexpr (!kSafe) {
             // 2^24: some exponent exceeded the reference by more than ~19
 #pragma unroll
             for (int r = 0; r < RB; ++r) bad = bad || l_tile[r] > 16777216.f;
@@ -607,8 +606,8 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
     };
 
     // One complete walk over the tile list.  The optimistic walk (kSafe = false) takes each
-    // row's reference from the unmasked scores of the first tile and never moves it on phase A
-    // tiles; it reports when that went wrong -- an exponent far above the reference (tile sum
+    // row's reference from the unmasked scores of the first tile and never moves it; it
+    // reports when that went wrong -- an exponent far above the reference (tile sum
     // above 2^24) or a row sum so small that the reference was far too high -- and the
     // workgroup then repeats the walk in the safe form, which moves the reference before the
     // probabilities of every tile (the textbook online soft-max, still with the lazy
