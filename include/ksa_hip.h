@@ -104,6 +104,24 @@ int ksa_copy_rows(const void* src, void* dst, const int32_t* src_index,
                   int heads, int D, const int64_t* src_strides, const int64_t* dst_strides,
                   void* stream);
 
+/* Pre-attention step: per-head RMSNorm of q and k, rotary embedding, layout write of q, k, v.
+ * Replaces HF:660-666 (q_norm / k_norm = Qwen3RMSNorm HF:64-79 on head_dim, the three
+ * .transpose(1, 2), apply_rotary_pos_emb HF:523-554 in its rotate_half form) and the
+ * .transpose(1, 2).contiguous() copies in front of the attention call, with the rounding
+ * points of the reference's 16-bit tensor ops.
+ *   q [batch, S, Hq, D], k, v [batch, S, Hkv, D]: projection outputs, strides {batch, row, head}
+ *   q_weight, k_weight [D]; cos, sin [batch or 1, S, D] with cos_strides {batch, row}
+ *   q_out, k_out, v_out: any {batch, row, head} strides -- the [batch, S, H, D] layout of
+ *   ksa_prefill_fwd, or rows of a [batch, H, capacity, D] cache tensor (pointer at the
+ *   first destination row).  q_out may alias q, k_out k, v_out v (same strides). */
+int ksa_pre_attention(const void* q, const void* k, const void* v, const void* q_weight,
+                      const void* k_weight, const void* cos, const void* sin, void* q_out,
+                      void* k_out, void* v_out, int batch, int S, int Hq, int Hkv, int D, int dtype,
+                      const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                      const int64_t* q_out_strides, const int64_t* k_out_strides,
+                      const int64_t* v_out_strides, const int64_t* cos_strides, float eps,
+                      void* stream);
+
 /* Host-side diagnostic: number of key columns in [a, b) visible to query row q under the
  * closed-form rule the kernels use (no GPU involved). */
 long long ksa_debug_count_visible(long long q, long long a, long long b, int C, int S, int W,

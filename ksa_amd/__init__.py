@@ -1,7 +1,8 @@
 """ksa_amd — MI355X (gfx950) kernels for the two attention hot paths of Kwai Summary
-Attention: the block-sparse prefill forward and decode over the ring-buffer KV cache.
+Attention: the block-sparse prefill forward and decode over the ring-buffer KV cache,
+plus the fused pre-attention step (q/k RMSNorm + rotary embedding + layout write) in front of them.
 
-Importing the package loads libksa_hip.so (built by `python -m ksa_amd.build`); if it is
+Importing the package loads libksa_hip.so (built by `python ksa_amd/build.py`); if it is
 missing the import fails — there is no other execution path.
 """
 from ._lib import KsaError, lib as _load
@@ -11,8 +12,9 @@ _load()
 from .prefill import SUMMARY_ATTN_CACHE, compute_block_sparsity, summary_attn_func  # noqa: E402
 from .decode import decode_attention_forward, ksa_decode  # noqa: E402
 from .cache import Qwen3RingBufferCache  # noqa: E402
+from .pre import pre_attention  # noqa: E402
 
 __all__ = [
     "KsaError", "SUMMARY_ATTN_CACHE", "compute_block_sparsity", "summary_attn_func",
-    "decode_attention_forward", "ksa_decode", "Qwen3RingBufferCache",
+    "decode_attention_forward", "ksa_decode", "Qwen3RingBufferCache", "pre_attention",
 ]

@@ -29,6 +29,7 @@ _SIGNATURES = {
     "ksa_decode_fwd": (_int, [_vp] * 6 + [_int] * 8 + [_i64p] * 4
                        + [ctypes.c_float, _int, _vp, ctypes.c_size_t, _vp]),
     "ksa_copy_rows": (_int, [_vp] * 4 + [_int] * 6 + [_i64p] * 2 + [_vp]),
+    "ksa_pre_attention": (_int, [_vp] * 10 + [_int] * 6 + [_i64p] * 7 + [ctypes.c_float, _vp]),
     "ksa_debug_count_visible": (ctypes.c_longlong, [ctypes.c_longlong] * 3 + [_int] * 7),
 }
 
@@ -44,7 +45,7 @@ def lib():
     if _lib is None:
         if not os.path.exists(LIB_PATH):
             raise KsaError(
-                f"{LIB_PATH} is missing: build it with `python -m ksa_amd.build` "
+                f"{LIB_PATH} is missing: build it with `python ksa_amd/build.py` "
                 "(hipcc, gfx950); ksa_amd has no other execution path")
         L = ctypes.CDLL(LIB_PATH)
         for name, (res, args) in _SIGNATURES.items():

@@ -57,3 +57,26 @@ def decode_sdpa(q, k, v, g):
     ve = v[:, :, None].expand(b, Hkv, g, L, D).reshape(b, Hkv * g, L, D)
     out = F.scaled_dot_product_attention(q, ke, ve, attn_mask=None, dropout_p=0.0, is_causal=False)
     return out.transpose(1, 2).contiguous()
+
+
+def pre_attention(q, k, v, q_weight, k_weight, cos, sin, eps=1e-6):
+    """The reference's pre-attention sequence restated with torch CPU tensor ops in the input
+    dtype (examples/pretrain/hf_template/modeling_qwen3sa.py:64-79 Qwen3RMSNorm.forward,
+    :516-554 rotate_half / apply_rotary_pos_emb, :660-666 call site), for [b, S, H, D] inputs
+    (the reference holds them as [b, H, S, D]; every op here is element-wise over (b, S, H)).
+    Returns (q', k', v)."""
+    def rms(x, w):
+        dt = x.dtype
+        xf = x.to(torch.float32)
+        var = xf.pow(2).mean(-1, keepdim=True)
+        xf = xf * torch.rsqrt(var + eps)
+        return w * xf.to(dt)
+
+    def rot(x):
+        h = x.shape[-1] // 2
+        return torch.cat((-x[..., h:], x[..., :h]), dim=-1)
+
+    c = cos.unsqueeze(2)  # broadcast over heads
+    s = sin.unsqueeze(2)
+    qn, kn = rms(q, q_weight), rms(k, k_weight)
+    return qn * c + rot(qn) * s, kn * c + rot(kn) * s, v
