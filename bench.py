@@ -131,6 +131,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--skip-decode", action="store_true")
     ap.add_argument("--skip-prefill", action="store_true")
+    ap.add_argument("--skip-pre-attention", action="store_true",
+                    help="do not time the fused pre-attention step (q/k RMSNorm + rotary + layout write "
+                         "at the prefill shape, reported under 'pre_attention')")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one ksa_copy_rows of 1 GiB (a plain copy kernel of known size, "
                          "used to scale the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
@@ -247,6 +250,38 @@ def main():
                            "config": {"workload": result["decode"]["workload"]},
                            "roofline": result["decode"]["roofline"]})
         del kc, vc
+        torch.cuda.empty_cache()
+
+    # ------------------------------------------------------------------ pre-attention step
+    if not args.skip_pre_attention:
+        chunks = args.prefill_chunks
+        Sp = chunks * (C + S)
+        g = torch.Generator(device=dev).manual_seed(2)
+        qkv = torch.randn(1, Sp, (Hq + 2 * Hkv) * D, generator=g, device=dev).to(torch.bfloat16)
+        qp = qkv[..., : Hq * D].view(1, Sp, Hq, D)
+        kp = qkv[..., Hq * D: (Hq + Hkv) * D].view(1, Sp, Hkv, D)
+        vp = qkv[..., (Hq + Hkv) * D:].view(1, Sp, Hkv, D)
+        wq = torch.ones(D, dtype=torch.bfloat16, device=dev)
+        ang = torch.arange(Sp, device=dev, dtype=torch.float32)[:, None] * \
+            (1.0 / 10000.0 ** (torch.arange(0, D, 2, device=dev, dtype=torch.float32) / D))[None]
+        emb = torch.cat((ang, ang), dim=-1)
+        cosb, sinb = emb.cos().to(torch.bfloat16)[None], emb.sin().to(torch.bfloat16)[None]
+        qo, ko, vo = torch.empty_like(qp), torch.empty_like(kp), torch.empty_like(vp)
+
+        def pstep():
+            ksa_amd.pre_attention(qp, kp, vp, wq, wq, cosb, sinb, 1e-6, q_out=qo, k_out=ko, v_out=vo)
+
+        wall, dev_ms = time_region(pstep, args.steps, args.warmup)
+        us = dev_ms * 1e3 / args.steps
+        pbytes = 2 * Sp * (Hq + 2 * Hkv) * D * 2 + 2 * Sp * D * 2   # q, k, v in and out; cos, sin in
+        result["pre_attention"] = {
+            "workload": f"pre-attention {chunks} chunks (q/k RMSNorm + rotary + layout write), {Hq}/{Hkv} heads",
+            "us_per_step": us, "algorithmic_bytes": pbytes, "hbm_gbps": pbytes / (us * 1e-6) / 1e9,
+            "roofline": {"bound": "hbm", "achieved": pbytes / (us * 1e-6) / 1e9, "peak": PEAK_HBM_GBPS,
+                         "unit": "GB/s", "frac": pbytes / (us * 1e-6) / 1e9 / PEAK_HBM_GBPS, "traffic": None,
+                         "kernel": "ksa_pre_attention_kernel<bf16,128>"},
+        }
+        del qkv, qo, ko, vo, cosb, sinb, emb, ang
         torch.cuda.empty_cache()
 
     # ------------------------------------------------------------------ CPU baseline

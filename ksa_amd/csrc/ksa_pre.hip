@@ -46,102 +46,158 @@ struct PreCvt<KsaBf16> {
     static __device__ __forceinline__ uint16_t down(float f) {
         return __builtin_bit_cast(uint16_t, (__bf16)f);
     }
+    // two values rounded into one word (low, high) and back
+    static __device__ __forceinline__ uint32_t down2(float lo, float hi) { return KsaOps<KsaBf16>::pack2(lo, hi); }
+    static __device__ __forceinline__ float lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
+    static __device__ __forceinline__ float hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
 };
 template <>
 struct PreCvt<KsaF16> {
+    // Conversion instructions written out: with plain _Float16 casts the compiler may keep
+    // excess precision across a down/up pair, which would drop the rounding points.
     static __device__ __forceinline__ float up(uint16_t u) {
-        return (float)__builtin_bit_cast(_Float16, u);
+        float f;
+        asm("v_cvt_f32_f16 %0, %1" : "=v"(f) : "v"((uint32_t)u));
+        return f;
     }
     static __device__ __forceinline__ uint16_t down(float f) {
-        return __builtin_bit_cast(uint16_t, (_Float16)f);
+        uint32_t h;
+        asm("v_cvt_f16_f32 %0, %1" : "=v"(h) : "v"(f));
+        return (uint16_t)h;
     }
+    static __device__ __forceinline__ uint32_t down2(float lo, float hi) {
+        return (uint32_t)down(lo) | ((uint32_t)down(hi) << 16);
+    }
+    static __device__ __forceinline__ float lo(uint32_t w) { return up((uint16_t)(w & 0xffffu)); }
+    static __device__ __forceinline__ float hi(uint32_t w) { return up((uint16_t)(w >> 16)); }
 };
 
+// value of the lane `n` places further inside the same row of 16 lanes (cyclic)
+template <int N>
+__device__ __forceinline__ uint32_t pre_row_ror(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x120 + N, 0xf, 0xf, false);
+}
+
+// sum over the LPR lanes that hold one head row; every lane of the row gets the total
+template <int LPR>
+__device__ __forceinline__ float pre_row_sum(float ss) {
+    if constexpr (LPR == 16) {  // rotations inside a DPP row (16 lanes)
+        ss += __builtin_bit_cast(float, pre_row_ror<8>(__builtin_bit_cast(uint32_t, ss)));
+        ss += __builtin_bit_cast(float, pre_row_ror<4>(__builtin_bit_cast(uint32_t, ss)));
+        ss += __builtin_bit_cast(float, pre_row_ror<2>(__builtin_bit_cast(uint32_t, ss)));
+        ss += __builtin_bit_cast(float, pre_row_ror<1>(__builtin_bit_cast(uint32_t, ss)));
+    } else {
+#pragma unroll
+        for (int m = 1; m < LPR; m <<= 1) ss += __shfl_xor(ss, m);
+    }
+    return ss;
+}
+
+// One workgroup takes one token at a time (grid-stride over tokens); its four waves share
+// the token's head rows, RPW rows of one of q / k / v per wave instruction.  Which tensor a
+// wave instruction works on, the token's base addresses and the weights are wave-uniform
+// (scalar registers); a lane only adds its row's offset, so no index division or 64-bit
+// multiply sits in the inner loop, and cos / sin are fetched once per wave and token.
 template <typename T, int D>
 __global__ __launch_bounds__(256) void ksa_pre_attention_kernel(const PreParams p) {
     using C = PreCvt<T>;
     constexpr int LPR = D / 8;          // lanes per head row
     constexpr int RPW = 64 / LPR;       // head rows per wave instruction
     const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int sub = lane / LPR;         // which of the wave's rows
     const int t = lane % LPR;           // 16-byte chunk inside the row
-    const int H_all = p.Hq + 2 * p.Hkv;
-    const int G = (H_all + RPW - 1) / RPW;
-    const int64_t items = (int64_t)p.batch * p.S * G;
-    const int64_t wave0 = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
-    const int64_t nwaves = ((int64_t)gridDim.x * blockDim.x) >> 6;
+    const int Hn[3] = {p.Hq, p.Hkv, p.Hkv};
+    const int Gq = (p.Hq + RPW - 1) / RPW, Gk = (p.Hkv + RPW - 1) / RPW;
+    const int G = Gq + 2 * Gk;
+    const int ntok = p.batch * p.S;
+    // rotate_half: the first half of a row takes -z[j + D/2], the second half +z[j - D/2];
+    // the sign goes into the sine once per token
+    const uint32_t sgn_bits = t < LPR / 2 ? 0x80008000u : 0u;
+    float wqf[8], wkf[8];  // this lane's slice of the two weight vectors
+    {
+        const u32x4 wq = *reinterpret_cast<const u32x4*>(p.w[0] + 8 * t);
+        const u32x4 wk = *reinterpret_cast<const u32x4*>(p.w[1] + 8 * t);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            wqf[2 * i] = C::lo(wq[i]);
+            wqf[2 * i + 1] = C::hi(wq[i]);
+            wkf[2 * i] = C::lo(wk[i]);
+            wkf[2 * i + 1] = C::hi(wk[i]);
+        }
+    }
+    // element offset of this lane's row inside a wave instruction's block of rows
+    uint32_t lsrc[3], ldst[3];
+#pragma unroll
+    for (int w = 0; w < 3; ++w) {
+        lsrc[w] = (uint32_t)sub * (uint32_t)p.s_hs[w] + 8 * t;
+        ldst[w] = (uint32_t)sub * (uint32_t)p.d_hs[w] + 8 * t;
+    }
 
-    for (int64_t it = wave0; it < items; it += nwaves) {
-        const int g = (int)(it % G);
-        const int64_t tok = it / G;
-        const int s = (int)(tok % p.S);
-        const int b = (int)(tok / p.S);
-        const int hh = g * RPW + sub;
-        if (hh >= H_all) continue;  // the whole lane group has nothing to do (no exchange partner outside it)
-        const int which = hh < p.Hq ? 0 : (hh < p.Hq + p.Hkv ? 1 : 2);
-        const int h = which == 0 ? hh : (which == 1 ? hh - p.Hq : hh - p.Hq - p.Hkv);
-        const uint16_t* sp = p.src[which] + b * p.s_bs[which] + (int64_t)s * p.s_rs[which] + h * p.s_hs[which] + 8 * t;
-        uint16_t* dp = p.dst[which] + b * p.d_bs[which] + (int64_t)s * p.d_rs[which] + h * p.d_hs[which] + 8 * t;
-        const u32x4 raw = *reinterpret_cast<const u32x4*>(sp);
-        if (which == 2) {  // v: layout change only
-            *reinterpret_cast<u32x4*>(dp) = raw;
-            continue;
-        }
-        float x[8];
+    for (int tok = blockIdx.x; tok < ntok; tok += gridDim.x) {
+        const int b = tok / p.S;
+        const int s = tok - b * p.S;
+        const u32x4 craw = *reinterpret_cast<const u32x4*>(p.cos + b * p.c_bs + (int64_t)s * p.c_rs + 8 * t);
+        const u32x4 sraw = *reinterpret_cast<const u32x4*>(p.sin + b * p.c_bs + (int64_t)s * p.c_rs + 8 * t);
+        float cs[8], sn[8];  // unpacked once per token; the sine carries the rotate_half sign
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            x[2 * i] = C::up((uint16_t)(raw[i] & 0xffffu));
-            x[2 * i + 1] = C::up((uint16_t)(raw[i] >> 16));
+            cs[2 * i] = C::lo(craw[i]);
+            cs[2 * i + 1] = C::hi(craw[i]);
+            sn[2 * i] = C::lo(sraw[i] ^ sgn_bits);
+            sn[2 * i + 1] = C::hi(sraw[i] ^ sgn_bits);
         }
-        float ss = 0.f;
+        for (int gi = wave; gi < G; gi += 4) {
+            const int which = gi < Gq ? 0 : (gi < Gq + Gk ? 1 : 2);          // wave-uniform
+            const int h0 = (gi - (which == 0 ? 0 : (which == 1 ? Gq : Gq + Gk))) * RPW;
+            const uint16_t* sbase = p.src[which] + b * p.s_bs[which] + (int64_t)s * p.s_rs[which] + (int64_t)h0 * p.s_hs[which];
+            uint16_t* dbase = p.dst[which] + b * p.d_bs[which] + (int64_t)s * p.d_rs[which] + (int64_t)h0 * p.d_hs[which];
+            if (h0 + sub >= Hn[which]) continue;  // a whole lane group is idle: its exchange partners are idle too
+            const u32x4 raw = *reinterpret_cast<const u32x4*>(sbase + lsrc[which]);
+            uint16_t* dp = dbase + ldst[which];
+            if (which == 2) {  // v: layout change only
+                *reinterpret_cast<u32x4*>(dp) = raw;
+                continue;
+            }
+            float x[8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) ss = fmaf(x[i], x[i], ss);
+            for (int i = 0; i < 4; ++i) {
+                x[2 * i] = C::lo(raw[i]);
+                x[2 * i + 1] = C::hi(raw[i]);
+            }
+            float ss = 0.f;
 #pragma unroll
-        for (int m = 1; m < LPR; m <<= 1) ss += __shfl_xor(ss, m);
-        const float inv = rsqrtf(ss * (1.0f / D) + p.eps);
-        const u32x4 wraw = *reinterpret_cast<const u32x4*>(p.w[which] + 8 * t);
-        const uint16_t* cb = p.cos + b * p.c_bs + (int64_t)s * p.c_rs + 8 * t;
-        const uint16_t* sb = p.sin + b * p.c_bs + (int64_t)s * p.c_rs + 8 * t;
-        const u32x4 craw = *reinterpret_cast<const u32x4*>(cb);
-        const u32x4 sraw = *reinterpret_cast<const u32x4*>(sb);
-        // z = round(w * round(x * inv)), packed again for the exchange
-        u32x4 zp;
-        float z[8];
+            for (int i = 0; i < 8; ++i) ss = fmaf(x[i], x[i], ss);
+            ss = pre_row_sum<LPR>(ss);
+            const float inv = rsqrtf(ss * (1.0f / D) + p.eps);
+            // z = round(w * round(x * inv)), kept packed for the exchange
+            u32x4 zp;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const float w0 = C::up((uint16_t)(wraw[i] & 0xffffu)), w1 = C::up((uint16_t)(wraw[i] >> 16));
-            const uint16_t y0 = C::down(x[2 * i] * inv), y1 = C::down(x[2 * i + 1] * inv);
-            const uint16_t z0 = C::down(w0 * C::up(y0)), z1 = C::down(w1 * C::up(y1));
-            z[2 * i] = C::up(z0);
-            z[2 * i + 1] = C::up(z1);
-            zp[i] = (uint32_t)z0 | ((uint32_t)z1 << 16);
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t y = C::down2(x[2 * i] * inv, x[2 * i + 1] * inv);
+                const float w0 = which == 0 ? wqf[2 * i] : wkf[2 * i];
+                const float w1 = which == 0 ? wqf[2 * i + 1] : wkf[2 * i + 1];
+                zp[i] = C::down2(w0 * C::lo(y), w1 * C::hi(y));
+            }
+            u32x4 outp;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                uint32_t pp;  // the partner half of the row
+                if constexpr (LPR == 16) pp = pre_row_ror<8>(zp[i]);
+                else pp = (uint32_t)__shfl_xor((int)zp[i], LPR / 2);
+                const uint32_t zc = C::down2(C::lo(zp[i]) * cs[2 * i], C::hi(zp[i]) * cs[2 * i + 1]);
+                const uint32_t rs = C::down2(C::lo(pp) * sn[2 * i], C::hi(pp) * sn[2 * i + 1]);
+                outp[i] = C::down2(C::lo(zc) + C::lo(rs), C::hi(zc) + C::hi(rs));
+            }
+            *reinterpret_cast<u32x4*>(dp) = outp;
         }
-        // rotate_half: the first half of the row takes -z[j + D/2], the second half z[j - D/2]
-        u32x4 pp;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) pp[i] = (uint32_t)__shfl_xor((int)zp[i], LPR / 2);
-        const float sgn = t < LPR / 2 ? -1.f : 1.f;
-        u32x4 outp;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const float r0 = sgn * C::up((uint16_t)(pp[i] & 0xffffu)), r1 = sgn * C::up((uint16_t)(pp[i] >> 16));
-            const float c0 = C::up((uint16_t)(craw[i] & 0xffffu)), c1 = C::up((uint16_t)(craw[i] >> 16));
-            const float s0 = C::up((uint16_t)(sraw[i] & 0xffffu)), s1 = C::up((uint16_t)(sraw[i] >> 16));
-            const float a0 = C::up(C::down(z[2 * i] * c0)) + C::up(C::down(r0 * s0));
-            const float a1 = C::up(C::down(z[2 * i + 1] * c1)) + C::up(C::down(r1 * s1));
-            outp[i] = (uint32_t)C::down(a0) | ((uint32_t)C::down(a1) << 16);
-        }
-        *reinterpret_cast<u32x4*>(dp) = outp;
     }
 }
 
 template <typename T, int D>
 int launch_pre(const PreParams& p, hipStream_t stream) {
-    constexpr int RPW = 64 / (D / 8);
-    const int H_all = p.Hq + 2 * p.Hkv;
-    const int64_t items = (int64_t)p.batch * p.S * ((H_all + RPW - 1) / RPW);
-    int64_t blocks = (items + 3) / 4;                    // 4 waves per block, one item per wave
-    const int64_t cap = 256 * 32;                        // grid-stride beyond that
+    int64_t blocks = (int64_t)p.batch * p.S;             // one token per workgroup pass
+    const int64_t cap = 256 * 16;                        // grid-stride beyond that
     if (blocks > cap) blocks = cap;
     hipLaunchKernelGGL((ksa_pre_attention_kernel<T, D>), dim3((unsigned)blocks), dim3(256), 0, stream, p);
     return ksa_check_launch();
@@ -162,6 +218,10 @@ extern "C" int ksa_pre_attention(const void* q, const void* k, const void* v, co
         !cos_strides)
         return KSA_ERR_NULL;
     if (batch <= 0 || S <= 0 || Hq <= 0 || Hkv <= 0 || !(eps >= 0.f)) return KSA_ERR_INVALID;
+    if ((int64_t)batch * S >= (1ll << 31)) return KSA_ERR_INVALID;
+    // a lane's row offset inside one wave instruction (at most 8 head rows) is kept in 32 bits
+    for (const int64_t* s3 : {q_strides, k_strides, v_strides, q_out_strides, k_out_strides, v_out_strides})
+        if (s3[2] < 0 || s3[2] * 8 + 128 >= (1ll << 32)) return KSA_ERR_INVALID;
     if (dtype != KSA_DTYPE_BF16 && dtype != KSA_DTYPE_F16) return KSA_ERR_UNSUPPORTED;
     if (D != 64 && D != 128) return KSA_ERR_UNSUPPORTED;
     const void* ptrs[] = {q, k, v, q_weight, k_weight, cos, sin, q_out, k_out, v_out};
