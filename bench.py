@@ -275,7 +275,8 @@ def main():
         us = dev_ms * 1e3 / args.steps
         pbytes = 2 * Sp * (Hq + 2 * Hkv) * D * 2 + 2 * Sp * D * 2   # q, k, v in and out; cos, sin in
         result["pre_attention"] = {
-            "workload": f"pre-attention {chunks} chunks (q/k RMSNorm + rotary + layout write), {Hq}/{Hkv} heads",
+            "workload": f"pre-attention-{chunks}-chunks-{Hq}q{Hkv}kv",
+            "what": "q/k RMSNorm on head_dim + rotary embedding + write of q, k, v in the attention layout",
             "us_per_step": us, "algorithmic_bytes": pbytes, "hbm_gbps": pbytes / (us * 1e-6) / 1e9,
             "roofline": {"bound": "hbm", "achieved": pbytes / (us * 1e-6) / 1e9, "peak": PEAK_HBM_GBPS,
                          "unit": "GB/s", "frac": pbytes / (us * 1e-6) / 1e9 / PEAK_HBM_GBPS, "traffic": None,
@@ -307,6 +308,8 @@ def main():
                 result["roofline"]["traffic"] = t.get("prefill_bytes_per_launch")
             if "decode" in result and result["decode"]["workload"] == t.get("decode_workload"):
                 result["decode"]["roofline"]["traffic"] = t.get("decode_bytes_per_launch")
+            if "pre_attention" in result and t.get("pre_attention_workload") == result["pre_attention"]["workload"]:
+                result["pre_attention"]["roofline"]["traffic"] = t.get("pre_attention_bytes_per_launch")
         except Exception:
             pass
     print(json.dumps(result))
