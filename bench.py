@@ -66,6 +66,47 @@ def time_region(fn, steps, warmup):
     return t1 - t0, e0.elapsed_time(e1)
 
 
+def sustained_rate(fn, flop_per_call, seconds, batch):
+    """Calls `fn` back to back for `seconds`; returns (TFLOP/s over the second half, mean shader
+    clock in MHz over the second half as rocm-smi reports it, or None)."""
+    import re
+    import subprocess
+    import threading
+    import torch
+    clocks, stop = [], threading.Event()
+
+    def sample():
+        while not stop.is_set():
+            try:
+                r = subprocess.run(["rocm-smi", "-c", "--csv"], capture_output=True, text=True, timeout=5)
+                m = re.search(r"\((\d+)Mhz\),\d+\s*$", r.stdout.strip().splitlines()[-1])
+                if m:
+                    clocks.append((time.perf_counter(), int(m.group(1))))
+            except Exception:
+                return
+            stop.wait(0.2)
+
+    th = threading.Thread(target=sample, daemon=True)
+    th.start()
+    t0 = time.perf_counter()
+    n = n_half = 0
+    t_half = None
+    while True:
+        for _ in range(batch):
+            fn()
+        torch.cuda.synchronize()
+        n += batch
+        t = time.perf_counter()
+        if t_half is None and t - t0 >= seconds / 2:
+            t_half, n_half = t, n
+        if t - t0 >= seconds and t_half is not None and n > n_half:
+            break
+    stop.set()
+    th.join()
+    late = [c for ts, c in clocks if ts >= t_half]
+    return flop_per_call * (n - n_half) / (t - t_half) / 1e12, (sum(late) / len(late) if late else None)
+
+
 def cpu_baseline_prefill(chunks, Hq, Hkv, D, C, S, W, tiles_per_mtile, budget_s=20.0):
     """The reference's CPU path (block mode, restated in oracle/cpu_path.py) on a bounded
     sample of 4096-row query blocks; rate in the same non-empty-block TFLOP/s unit."""
@@ -134,6 +175,13 @@ def main():
     ap.add_argument("--skip-pre-attention", action="store_true",
                     help="do not time the fused pre-attention step (q/k RMSNorm + rotary + layout write "
                          "at the prefill shape, reported under 'pre_attention')")
+    ap.add_argument("--sustain", type=float, default=0.0, metavar="SECONDS",
+                    help="also loop the prefill launch for SECONDS and report the rate of the second "
+                         "half under 'sustained' (the chip lowers its clock under a long MFMA load)")
+    ap.add_argument("--mfma-ceiling", type=float, default=0.0, metavar="SECONDS",
+                    help="also time a pure bf16 MFMA instruction stream for SECONDS with random and "
+                         "with all-zero operands (second-half rate, 'mfma_stream'): the rate the "
+                         "power limit allows, to read the prefill rate against")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one ksa_copy_rows of 1 GiB (a plain copy kernel of known size, "
                          "used to scale the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
@@ -205,8 +253,29 @@ def main():
                          "traffic": None, "kernel": "ksa_prefill_kernel<bf16,128>",
                          "kernel_ms": kern_ms},
         })
+        if args.sustain > 0:
+            rate, clk = sustained_rate(step, flops, args.sustain, 10)
+            result["sustained"] = {"seconds": args.sustain, "tflops_second_half": rate,
+                                   "frac_of_peak": rate / PEAK_BF16_TFLOPS, "sclk_mhz_mean": clk}
         del q, k, v, sp
         torch.cuda.empty_cache()
+
+    if args.mfma_ceiling > 0:
+        import ctypes
+        L = _lib.lib()
+        out = torch.empty(256 * 8 * 64, dtype=torch.float32, device=dev)
+        fl = ctypes.c_double(0.0)
+        res = {}
+        for name, zero in (("random_operands", 0), ("zero_operands", 1)):
+            def mstep():
+                _lib.check(L.ksa_probe_mfma_stream(out.data_ptr(), 256, 8, 2000, zero, ctypes.byref(fl),
+                                                   _lib.stream_ptr(dev)), "ksa_probe_mfma_stream")
+            mstep()
+            torch.cuda.synchronize()
+            rate, clk = sustained_rate(mstep, fl.value, args.mfma_ceiling, 10)
+            res[name] = {"tflops_second_half": rate, "frac_of_peak": rate / PEAK_BF16_TFLOPS,
+                         "sclk_mhz_mean": clk}
+        result["mfma_stream"] = {"seconds_each": args.mfma_ceiling, "waves_per_simd": 2, **res}
 
     # ------------------------------------------------------------------ decode
     if not args.skip_decode:

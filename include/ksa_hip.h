@@ -122,6 +122,14 @@ int ksa_pre_attention(const void* q, const void* k, const void* v, const void* q
                       const int64_t* v_out_strides, const int64_t* cos_strides, float eps,
                       void* stream);
 
+/* Measurement aid (no counterpart in the reference): launches a pure stream of bf16 MFMA
+ * 32x32x16 instructions (blocks x waves_per_block waves, 16 * iters instructions each, operands
+ * random or all zero) and returns the floating-point operations of the launch in *flop.  Timed
+ * over seconds it gives the MFMA rate the chip sustains under its power limit, against which
+ * the prefill kernel's rate can be read.  out: device float[blocks * waves_per_block * 64]. */
+int ksa_probe_mfma_stream(void* out, int blocks, int waves_per_block, int iters,
+                          int zero_operands, double* flop, void* stream);
+
 /* Host-side diagnostic: number of key columns in [a, b) visible to query row q under the
  * closed-form rule the kernels use (no GPU involved). */
 long long ksa_debug_count_visible(long long q, long long a, long long b, int C, int S, int W,

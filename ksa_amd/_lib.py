@@ -30,6 +30,7 @@ _SIGNATURES = {
                        + [ctypes.c_float, _int, _vp, ctypes.c_size_t, _vp]),
     "ksa_copy_rows": (_int, [_vp] * 4 + [_int] * 6 + [_i64p] * 2 + [_vp]),
     "ksa_pre_attention": (_int, [_vp] * 10 + [_int] * 6 + [_i64p] * 7 + [ctypes.c_float, _vp]),
+    "ksa_probe_mfma_stream": (_int, [_vp] + [_int] * 4 + [ctypes.POINTER(ctypes.c_double), _vp]),
     "ksa_debug_count_visible": (ctypes.c_longlong, [ctypes.c_longlong] * 3 + [_int] * 7),
 }
 
