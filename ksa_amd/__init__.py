@@ -1,6 +1,7 @@
 """ksa_amd — MI355X (gfx950) kernels for the two attention hot paths of Kwai Summary
 Attention: the block-sparse prefill forward and decode over the ring-buffer KV cache,
-plus the fused pre-attention step (q/k RMSNorm + rotary embedding + layout write) in front of them.
+plus the fused pre-attention step (q/k RMSNorm + rotary embedding + layout write) in front of them
+and the end-to-end decoder (`model`) that calls all of them.
 
 Importing the package loads libksa_hip.so (built by `python ksa_amd/build.py`); if it is
 missing the import fails — there is no other execution path.
@@ -13,8 +14,10 @@ from .prefill import SUMMARY_ATTN_CACHE, compute_block_sparsity, summary_attn_fu
 from .decode import decode_attention_forward, ksa_decode  # noqa: E402
 from .cache import Qwen3RingBufferCache  # noqa: E402
 from .pre import pre_attention  # noqa: E402
+from .model import KsaQwen3Config, KsaQwen3ForCausalLM, init_weights  # noqa: E402
 
 __all__ = [
     "KsaError", "SUMMARY_ATTN_CACHE", "compute_block_sparsity", "summary_attn_func",
     "decode_attention_forward", "ksa_decode", "Qwen3RingBufferCache", "pre_attention",
+    "KsaQwen3Config", "KsaQwen3ForCausalLM", "init_weights",
 ]

@@ -138,6 +138,49 @@ class Qwen3RingBufferCache:
         n = self._text_len[layer_idx]
         return self.key_cache[layer_idx][:, :, :n, :], self.value_cache[layer_idx][:, :, :n, :]
 
+    def prefill_slots(self, layer_idx: int, bsz: int, heads: int, n: int, D: int, dtype, device,
+                      n_summary: int = 0):
+        """`update` without the copy: reserves `n` rows for prefill K/V and returns the two
+        [bsz, n, heads, D] views of them for the producer to write (e.g. the pre-attention
+        kernel).  Same counters as `update` with a summary mask holding `n_summary` rows."""
+        cur = self._text_len[layer_idx]
+        need = cur + n
+        if self.key_cache[layer_idx] is None:
+            cap = need + self._APPEND_HEADROOM
+            self.key_cache[layer_idx] = torch.empty(bsz, heads, cap, D, dtype=dtype, device=device)
+            self.value_cache[layer_idx] = torch.empty(bsz, heads, cap, D, dtype=dtype, device=device)
+            self._capacity[layer_idx] = cap
+        elif need > self._capacity[layer_idx]:
+            self._regrow(layer_idx, max(need + self._APPEND_HEADROOM, 2 * self._capacity[layer_idx]), cur)
+        self._text_len[layer_idx] = need
+        if self.summary_chunk_size > 0:
+            self.cur_chunk_sizes[layer_idx] += n
+            self.true_tokens[layer_idx] += n - n_summary
+        return (self.key_cache[layer_idx][:, :, cur:need, :].transpose(1, 2),
+                self.value_cache[layer_idx][:, :, cur:need, :].transpose(1, 2))
+
+    def text_slots(self, layer_idx: int, bsz: int, heads: int, D: int, dtype, device):
+        """`update_text` without the copy: returns the [bsz, 1, heads, D] views of the row the
+        next text token's K/V belong in and advances the counters."""
+        if self.is_large_window[layer_idx]:
+            row = self._text_len[layer_idx]
+            if self.key_cache[layer_idx] is None:
+                cap = row + 1 + self._APPEND_HEADROOM
+                self.key_cache[layer_idx] = torch.empty(bsz, heads, cap, D, dtype=dtype, device=device)
+                self.value_cache[layer_idx] = torch.empty(bsz, heads, cap, D, dtype=dtype, device=device)
+                self._capacity[layer_idx] = cap
+            elif row + 1 > self._capacity[layer_idx]:
+                self._regrow(layer_idx, max(row + 1 + self._APPEND_HEADROOM, 2 * self._capacity[layer_idx]), row)
+            self._text_len[layer_idx] = row + 1
+        else:
+            cbl = self._chunk_buf_len[layer_idx]
+            row = self.summary_token_num + self.summary_chunk_size - 1 - cbl
+            self._chunk_buf_len[layer_idx] = cbl + 1
+        self.cur_chunk_sizes[layer_idx] += 1
+        self.true_tokens[layer_idx] += 1
+        return (self.key_cache[layer_idx][:, :, row:row + 1, :].transpose(1, 2),
+                self.value_cache[layer_idx][:, :, row:row + 1, :].transpose(1, 2))
+
     def reorganize_after_prefill(self, summary_mask: torch.Tensor):
         """Prefill order -> ring layout for every layer.  summary_mask: bool [bsz, prefill_len]."""
         if self._reorganized:

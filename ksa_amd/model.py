@@ -1,0 +1,352 @@
+"""End-to-end KSA decoder (Qwen3 shape with Summary Attention) on the MI355X kernels.
+
+The caller of both hot paths, restated from the reference's inference model
+(examples/pretrain/hf_template/modeling_qwen3sa.py): `Qwen3Model.forward` :1203-1324 (expand the
+prompt with summary tokens, run the layers, reorganise the cache after prefill, drop the summary
+rows), `_expand_input_with_summary_tokens` :1080-1177, `Qwen3DecoderLayer.forward` :905-953,
+`Qwen3SummaryAttention.forward` :741-880 (prefill / one-token decode / chunk-boundary decode),
+`Qwen3MLP` :507-514, `Qwen3RMSNorm` :64-79, `Qwen3RotaryEmbedding` :975-1032,
+`Qwen3ForCausalLM.forward` :1343-1420 (logits of the last position, truncated to the text
+vocabulary) and `prepare_inputs_for_generation` :1432-1560 (what a decode step feeds: the new
+token, plus the summary tokens when the chunk completes, and their position ids).
+
+Differences from the reference, on purpose:
+* any batch size (the reference refuses batch > 1 at :753; its cache tensors and counters are
+  already batch-shaped, all sequences of a batch have the same length);
+* weights are plain tensors (fused q|k|v and gate|up matrices), not nn.Modules; projections and
+  the MLP are torch matmuls (hipBLASLt), everything attention-side is this package's kernels;
+* a "full attention" layer is, as in the reference's inference model, a Summary layer whose
+  window is larger than any sequence (append-only text cache, :114-115, :232-242);
+* `summary_independent_parameters` is supported for mix_coeff 0 and 1 (the reference's default
+  1.0, :765-791): the summary rows then take their q, k, v from their own projection.
+
+The attention-side operators come from an `ops` object; the default binds the HIP kernels of this
+package and needs a GPU.  Tests pass a CPU fp32 implementation of the same four operators to
+obtain the reference run of this very module.
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass, field
+from typing import List, Optional, Tuple, Union
+
+import torch
+import torch.nn.functional as F
+
+
+@dataclass
+class KsaQwen3Config:
+    """Field names follow the reference's config.json (examples/pretrain/hf_template/config.json)."""
+    hidden_size: int = 2560
+    num_hidden_layers: int = 36
+    num_attention_heads: int = 32
+    num_key_value_heads: int = 8
+    head_dim: int = 128
+    intermediate_size: int = 9728
+    rms_norm_eps: float = 1e-6
+    rope_theta: float = 1e6
+    vocab_size: int = 151936
+    initializer_range: float = 0.02
+    tie_word_embeddings: bool = True
+    summary_chunk_size: int = 128
+    summary_token_num: int = 8
+    summary_token_begin: int = 151936          # ids of the summary tokens: begin .. begin + num - 1
+    # per layer; the reference writes this as a pattern string such as "([4]*3+[1024]*1)*9".
+    # As in the reference's cache (:114-115) there are two kinds of layers: those with the
+    # smallest window, and "large window" layers (anything larger), which keep every text row
+    # and no summaries during decoding.
+    summary_sliding_chunk_num: Union[int, List[int]] = field(
+        default_factory=lambda: ([4] * 3 + [1 << 20]) * 9)
+    summary_chunk_position_ids_type: str = "origin"
+    summary_token_position_ids_type: str = "last_chunk_slice_right"
+    summary_independent_parameters: bool = False
+    mix_coeff: float = 1.0
+
+    def sliding_chunk_nums(self) -> List[int]:
+        v = self.summary_sliding_chunk_num
+        if isinstance(v, int):
+            return [v] * self.num_hidden_layers
+        v = [int(x) for x in v]
+        if len(v) != self.num_hidden_layers:
+            raise ValueError(f"summary_sliding_chunk_num has {len(v)} entries for "
+                             f"{self.num_hidden_layers} layers")
+        return v
+
+    def embedding_rows(self) -> int:
+        return max(self.vocab_size, self.summary_token_begin + self.summary_token_num)
+
+
+def init_weights(config: KsaQwen3Config, device, dtype=torch.bfloat16, seed: int = 0) -> dict:
+    """Random weights as the reference initialises them (normal, std = initializer_range, for
+    every Linear and Embedding; RMSNorm weights 1), drawn on `device` tensor by tensor and rounded
+    to `dtype`."""
+    g = torch.Generator(device=device).manual_seed(seed)
+    std = config.initializer_range
+    H, D = config.hidden_size, config.head_dim
+    nq, nkv, I = config.num_attention_heads * D, config.num_key_value_heads * D, config.intermediate_size
+
+    def normal(*shape):
+        return (torch.randn(*shape, generator=g, device=device, dtype=torch.float32) * std).to(dtype)
+
+    def ones(n):
+        return torch.ones(n, device=device, dtype=dtype)
+
+    layers = []
+    for _ in range(config.num_hidden_layers):
+        lw = {
+            "input_layernorm": ones(H), "post_attention_layernorm": ones(H),
+            "qkv_proj": normal(nq + 2 * nkv, H),        # rows: q | k | v
+            "q_norm": ones(D), "k_norm": ones(D),
+            "o_proj": normal(H, nq),
+            "gate_up_proj": normal(2 * I, H),           # rows: gate | up
+            "down_proj": normal(H, I),
+        }
+        if config.summary_independent_parameters:
+            lw["qkv_proj_summary"] = normal(nq + 2 * nkv, H)
+        layers.append(lw)
+    w = {"embed_tokens": normal(config.embedding_rows(), H), "layers": layers, "norm": ones(H)}
+    if not config.tie_word_embeddings:
+        w["lm_head"] = normal(config.vocab_size, H)
+    return w
+
+
+def convert_weights(weights: dict, device, dtype) -> dict:
+    """The same weights on another device / in another dtype (e.g. the fp32 CPU copy of a bf16 set)."""
+    def conv(x):
+        if isinstance(x, torch.Tensor):
+            return x.to(device=device, dtype=dtype)
+        if isinstance(x, dict):
+            return {k: conv(v) for k, v in x.items()}
+        if isinstance(x, list):
+            return [conv(v) for v in x]
+        return x
+    return conv(weights)
+
+
+class HipOps:
+    """The attention-side operators of the model, bound to this package's HIP kernels."""
+
+    def __init__(self):
+        from . import cache, decode, pre, prefill
+        self.cache_cls = cache.Qwen3RingBufferCache
+        self.pre_attention = pre.pre_attention
+        self.summary_attn_func = prefill.summary_attn_func
+        self._decode = decode.ksa_decode
+
+    def decode(self, q, kbuf, vbuf, start, end, scale):
+        return self._decode(q, kbuf, vbuf, start, end, scale=scale)
+
+
+def expand_with_summary_tokens(input_ids: torch.Tensor, config: KsaQwen3Config):
+    """Prompt -> (ids with `summary_token_num` summary ids after every complete chunk, position
+    ids [1, L], summary mask [L]).  Text keeps its original positions ('origin'); summary token k
+    (1-based, 'last_chunk_slice_right') of chunk i sits at i*C + (k*C)//S - 1, token k-1 of
+    'last_chunk_slice_left' at max(i*C, i*C + ((k-1)*C)//S - 1); 'zeros' and 'inner_chunk' as in
+    the reference (:1134-1175)."""
+    C, S = config.summary_chunk_size, config.summary_token_num
+    bsz, n = input_ids.shape
+    dev = input_ids.device
+    n_full, rem = divmod(n, C)
+    blk = C + S
+    L = n_full * blk + rem
+    slot = torch.arange(L, device=dev)
+    chunk, off = slot // blk, slot % blk
+    is_sum = off >= C
+    text_src = chunk * C + torch.clamp(off, max=C - 1)
+    ids = input_ids[:, text_src]
+    sum_ids = (config.summary_token_begin + (off - C)).to(input_ids.dtype)
+    ids = torch.where(is_sum[None], sum_ids[None].expand(bsz, -1), ids)
+
+    if config.summary_chunk_position_ids_type == "origin":
+        text_pos = text_src
+    elif config.summary_chunk_position_ids_type == "inner_chunk":
+        text_pos = torch.clamp(off, max=C - 1)
+    else:
+        raise ValueError(f"summary_chunk_position_ids_type {config.summary_chunk_position_ids_type!r}")
+    kind = config.summary_token_position_ids_type
+    if kind == "zeros":
+        sum_pos = torch.zeros_like(slot)
+    elif kind in ("last_chunk_slice_left", "last_chunk_slice_right"):
+        k = (off - C) + (1 if kind == "last_chunk_slice_right" else 0)
+        sum_pos = torch.maximum(chunk * C + (k * C) // S - 1, chunk * C)
+    else:
+        raise ValueError(f"summary_token_position_ids_type {kind!r}")
+    pos = torch.where(is_sum, sum_pos, text_pos)
+    return ids, pos[None], is_sum
+
+
+def boundary_position_ids(true_tokens: int, config: KsaQwen3Config, device) -> torch.Tensor:
+    """Position ids [1, 1 + S] of a chunk-boundary decode step: the text token at its index in
+    the text, the summary tokens by the same slice rule as in prefill (:1497-1531)."""
+    C, S = config.summary_chunk_size, config.summary_token_num
+    kind = config.summary_token_position_ids_type
+    if config.summary_chunk_position_ids_type == "origin":
+        text = true_tokens
+    elif config.summary_chunk_position_ids_type == "inner_chunk":
+        text = C - 1
+    else:
+        raise ValueError(f"summary_chunk_position_ids_type {config.summary_chunk_position_ids_type!r}")
+    prev_end = true_tokens + 1 - C
+    if kind == "zeros":
+        sp = torch.zeros(S, dtype=torch.long, device=device)
+    elif kind in ("last_chunk_slice_left", "last_chunk_slice_right"):
+        k = torch.arange(S, device=device, dtype=torch.long) + (1 if kind == "last_chunk_slice_right" else 0)
+        sp = torch.clamp(prev_end + (k * C) // S - 1, min=prev_end)
+    else:
+        raise ValueError(f"summary_token_position_ids_type {kind!r}")
+    return torch.cat([torch.tensor([text], dtype=torch.long, device=device), sp])[None]
+
+
+class KsaQwen3ForCausalLM:
+    """Inference-only decoder: `forward` for one prefill or one decode step, `generate` for a
+    greedy loop.  All sequences of a batch have the same length."""
+
+    def __init__(self, config: KsaQwen3Config, weights: dict, ops=None):
+        self.config = config
+        self.w = weights
+        self.ops = ops if ops is not None else HipOps()
+        if config.summary_independent_parameters and config.mix_coeff not in (0, 0.0, 1, 1.0):
+            raise NotImplementedError("summary_independent_parameters needs mix_coeff 0 or 1")
+        self.scns = config.sliding_chunk_nums()
+        D = config.head_dim
+        self.inv_freq = 1.0 / (config.rope_theta ** (torch.arange(0, D, 2, dtype=torch.int64).float() / D))
+        self.scaling = D ** -0.5
+        emb = weights["embed_tokens"]
+        self.dtype, self.device = emb.dtype, emb.device
+        self.lm_head = emb[: config.vocab_size] if config.tie_word_embeddings else weights["lm_head"]
+
+    # ---- pieces ----------------------------------------------------------------------
+    def _rms(self, x, w):
+        xf = x.float()
+        xf = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + self.config.rms_norm_eps)
+        return w * xf.to(x.dtype)
+
+    def _rope_tables(self, position_ids):
+        """cos, sin [1, L, D] in the model dtype from position ids [1, L] (computed in fp32)."""
+        freqs = position_ids[0].to(self.device).float()[:, None] * self.inv_freq.to(self.device)[None, :]
+        emb = torch.cat((freqs, freqs), dim=-1)
+        return emb.cos().to(self.dtype)[None], emb.sin().to(self.dtype)[None]
+
+    def _qkv(self, lw, h, summary_rows):
+        """Projection outputs as strided views q [b, L, Hq, D], k, v [b, L, Hkv, D]."""
+        cfg = self.config
+        D, Hq, Hkv = cfg.head_dim, cfg.num_attention_heads, cfg.num_key_value_heads
+        qkv = F.linear(h, lw["qkv_proj"])
+        if (cfg.summary_independent_parameters and cfg.mix_coeff != 0 and summary_rows is not None
+                and summary_rows.numel() > 0):
+            qkv[:, summary_rows] = F.linear(h[:, summary_rows], lw["qkv_proj_summary"])
+        b, L, _ = qkv.shape
+        q = qkv[..., : Hq * D].view(b, L, Hq, D)
+        k = qkv[..., Hq * D: (Hq + Hkv) * D].view(b, L, Hkv, D)
+        v = qkv[..., (Hq + Hkv) * D:].view(b, L, Hkv, D)
+        return q, k, v
+
+    def _mlp(self, lw, x):
+        gu = F.linear(x, lw["gate_up_proj"])
+        I = self.config.intermediate_size
+        return F.linear(F.silu(gu[..., :I]) * gu[..., I:], lw["down_proj"])
+
+    def _logits(self, hidden_last):
+        return F.linear(self._rms(hidden_last, self.w["norm"]), self.lm_head)
+
+    # ---- prefill ---------------------------------------------------------------------
+    @torch.no_grad()
+    def prefill(self, input_ids: torch.Tensor):
+        """input_ids [b, n] -> (logits [b, 1, vocab] of the last prompt token, cache)."""
+        cfg, ops = self.config, self.ops
+        C, S = cfg.summary_chunk_size, cfg.summary_token_num
+        ids, pos, is_sum = expand_with_summary_tokens(input_ids.to(self.device), cfg)
+        b, L = ids.shape
+        n_sum = int(is_sum.sum().item())
+        sum_rows = torch.nonzero(is_sum).flatten()
+        cos, sin = self._rope_tables(pos)
+        cache = ops.cache_cls(cfg, self.scns)
+        x = self.w["embed_tokens"][ids]
+        Hkv, D = cfg.num_key_value_heads, cfg.head_dim
+        for li, lw in enumerate(self.w["layers"]):
+            h = self._rms(x, lw["input_layernorm"])
+            q, k, v = self._qkv(lw, h, sum_rows)
+            k_slot, v_slot = cache.prefill_slots(li, b, Hkv, L, D, self.dtype, self.device, n_sum)
+            q, k, v = ops.pre_attention(q, k, v, lw["q_norm"], lw["k_norm"], cos, sin, cfg.rms_norm_eps,
+                                        k_out=k_slot, v_out=v_slot)
+            attn, _ = ops.summary_attn_func(q, k, v, C, S, self.scns[li], summary_pos=is_sum)
+            x = x + F.linear(attn.reshape(b, L, -1), lw["o_proj"])
+            x = x + self._mlp(lw, self._rms(x, lw["post_attention_layernorm"]))
+        cache.reorganize_after_prefill(is_sum[None])
+        last_text = L - 1 if (L % (C + S)) != 0 else L - 1 - S   # the last prompt token's slot
+        return self._logits(x[:, last_text:last_text + 1])[..., : cfg.vocab_size], cache
+
+    # ---- decode ----------------------------------------------------------------------
+    @torch.no_grad()
+    def decode_step(self, token_ids: torch.Tensor, cache):
+        """token_ids [b, 1] (the newest text token) -> logits [b, 1, vocab].  When the token
+        completes a chunk the step also runs the chunk's summary tokens and stores their K/V."""
+        cfg, ops = self.config, self.ops
+        C, S = cfg.summary_chunk_size, cfg.summary_token_num
+        Hkv, D = cfg.num_key_value_heads, cfg.head_dim
+        b = token_ids.shape[0]
+        true_tokens = cache.get_true_token_num()
+        boundary = cache.get_cur_chunk_size() == C - 1
+        ids = token_ids.to(self.device)
+        if boundary:
+            sids = torch.arange(S, device=self.device, dtype=ids.dtype) + cfg.summary_token_begin
+            ids = torch.cat([ids, sids[None].expand(b, -1)], dim=1)
+            pos = boundary_position_ids(true_tokens, cfg, self.device)
+            sum_rows = torch.arange(1, 1 + S, device=self.device)
+        else:
+            p = true_tokens if cfg.summary_chunk_position_ids_type == "origin" else cache.get_cur_chunk_size()
+            pos = torch.tensor([[p]], dtype=torch.long, device=self.device)
+            sum_rows = None
+        cos, sin = self._rope_tables(pos)
+        x = self.w["embed_tokens"][ids]
+        for li, lw in enumerate(self.w["layers"]):
+            h = self._rms(x, lw["input_layernorm"])
+            q, k, v = self._qkv(lw, h, sum_rows)
+            if not boundary:
+                k_slot, v_slot = cache.text_slots(li, b, Hkv, D, self.dtype, self.device)
+                q, _, _ = ops.pre_attention(q, k, v, lw["q_norm"], lw["k_norm"], cos, sin, cfg.rms_norm_eps,
+                                            k_out=k_slot, v_out=v_slot)
+                a, e = cache.attention_range(li)
+                attn = ops.decode(q.transpose(1, 2), cache.key_cache[li], cache.value_cache[li], a, e,
+                                  self.scaling)
+            else:
+                q, k, v = ops.pre_attention(q, k, v, lw["q_norm"], lw["k_norm"], cos, sin, cfg.rms_norm_eps)
+                qh, kh, vh = q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2)
+                cache.update_text(kh[:, :, :1], vh[:, :, :1], li)
+                a, e = cache.attention_range(li)
+                text_out = ops.decode(qh[:, :, :1], cache.key_cache[li], cache.value_cache[li], a, e,
+                                      self.scaling)
+                k_cs, v_cs = cache.get_summary_attention_kv(li, kh[:, :, 1:], vh[:, :, 1:])
+                sum_out = ops.decode(qh[:, :, 1:], k_cs, v_cs, 0, k_cs.shape[2], self.scaling)
+                cache.update_summary(kh[:, :, 1:], vh[:, :, 1:], li)
+                attn = torch.cat([text_out, sum_out], dim=1)
+            x = x + F.linear(attn.reshape(b, ids.shape[1], -1), lw["o_proj"])
+            x = x + self._mlp(lw, self._rms(x, lw["post_attention_layernorm"]))
+        cache.reset_chunk_counter()
+        return self._logits(x[:, :1])[..., : cfg.vocab_size]
+
+    # ---- driver ----------------------------------------------------------------------
+    def forward(self, input_ids: torch.Tensor, cache=None):
+        """Prefill when there is no (or an empty) cache, one decode step otherwise."""
+        if cache is None or cache.get_seq_length() == 0:
+            return self.prefill(input_ids)
+        return self.decode_step(input_ids[:, -1:], cache), cache
+
+    @torch.no_grad()
+    def generate(self, input_ids: torch.Tensor, max_new_tokens: int, forced: Optional[torch.Tensor] = None,
+                 return_logits: bool = False):
+        """Greedy decoding.  Returns ids [b, n + max_new_tokens] (and the logits of every step,
+        [b, max_new_tokens, vocab], on request).  `forced` [b, max_new_tokens] replaces the
+        arg-max token fed back at every step (teacher forcing, for comparing two runs)."""
+        logits, cache = self.prefill(input_ids)
+        out, steps = [], []
+        for t in range(max_new_tokens):
+            if return_logits:
+                steps.append(logits[:, 0].float())
+            nxt = logits[:, 0].argmax(-1, keepdim=True)
+            out.append(nxt)
+            if t + 1 < max_new_tokens:
+                feed = nxt if forced is None else forced[:, t:t + 1].to(self.device)
+                logits = self.decode_step(feed, cache)
+        ids = torch.cat([input_ids.to(self.device)] + out, dim=1)
+        return (ids, torch.stack(steps, dim=1)) if return_logits else ids
