@@ -182,6 +182,14 @@ def main():
                     help="also time a pure bf16 MFMA instruction stream for SECONDS with random and "
                          "with all-zero operands (second-half rate, 'mfma_stream'): the rate the "
                          "power limit allows, to read the prefill rate against")
+    ap.add_argument("--e2e", action="store_true",
+                    help="also run the end-to-end decoder (random-init 4B shape: 36 layers, 3 Summary : 1 "
+                         "full, batch 8, 32k-token prompt, 256 greedy steps) and report prefill and "
+                         "decode tokens/s under 'e2e'")
+    ap.add_argument("--e2e-batch", type=int, default=8)
+    ap.add_argument("--e2e-prompt", type=int, default=32768)
+    ap.add_argument("--e2e-new", type=int, default=256)
+    ap.add_argument("--e2e-layers", type=int, default=36)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one ksa_copy_rows of 1 GiB (a plain copy kernel of known size, "
                          "used to scale the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
@@ -355,6 +363,42 @@ def main():
         torch.cuda.empty_cache()
 
     # ------------------------------------------------------------------ CPU baseline
+    if args.e2e:
+        from ksa_amd.model import KsaQwen3Config, KsaQwen3ForCausalLM, init_weights
+        nl = args.e2e_layers
+        cfg = KsaQwen3Config(num_hidden_layers=nl,
+                             summary_sliding_chunk_num=[(1 << 20) if i % 4 == 3 else W for i in range(nl)])
+        weights = init_weights(cfg, dev, torch.bfloat16, seed=0)
+        model = KsaQwen3ForCausalLM(cfg, weights)
+        gi = torch.Generator(device=dev).manual_seed(3)
+        ids = torch.randint(0, cfg.vocab_size, (args.e2e_batch, args.e2e_prompt), generator=gi, device=dev)
+        model.generate(ids[:, :300], 3)                 # library set-up (GEMM handles, index cache)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        logits, cache = model.prefill(ids)
+        torch.cuda.synchronize()
+        t_prefill = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        n_boundary = 0
+        for _ in range(args.e2e_new):
+            nxt = logits[:, 0].argmax(-1, keepdim=True)
+            n_boundary += cache.get_cur_chunk_size() == cfg.summary_chunk_size - 1
+            logits = model.decode_step(nxt, cache)
+        torch.cuda.synchronize()
+        t_decode = time.perf_counter() - t0
+        result["e2e"] = {
+            "workload": f"random-init decoder, {nl} layers (3 Summary W={W} : 1 unbounded window), hidden "
+                        f"{cfg.hidden_size}, {Hq}/{Hkv} heads, batch {args.e2e_batch}, prompt "
+                        f"{args.e2e_prompt}, {args.e2e_new} greedy steps",
+            "prefill_s": t_prefill, "prefill_tokens_per_s": args.e2e_batch * args.e2e_prompt / t_prefill,
+            "decode_s": t_decode, "decode_ms_per_step": t_decode / args.e2e_new * 1e3,
+            "decode_tokens_per_s": args.e2e_batch * args.e2e_new / t_decode,
+            "chunk_boundary_steps": int(n_boundary),
+            "hbm_allocated_gb": torch.cuda.max_memory_allocated() / 1e9,
+        }
+        del model, weights, cache, logits
+        torch.cuda.empty_cache()
+
     if not args.no_cpu_baseline:
         try:
             Sq_ = args.prefill_chunks * (C + S)
