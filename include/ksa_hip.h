@@ -122,6 +122,25 @@ int ksa_pre_attention(const void* q, const void* k, const void* v, const void* q
                       const int64_t* v_out_strides, const int64_t* cos_strides, float eps,
                       void* stream);
 
+/* Residual add + RMSNorm over the hidden size, one pass.
+ * Replaces Qwen3RMSNorm.forward (HF:64-79: fp32 normalisation, rounded to the 16-bit type, times
+ * the 16-bit weight) together with the residual add in front of it (HF:946, :952).
+ *   out_sum  = x + residual   (skipped when residual is null)
+ *   out_norm = weight * round(s * rsqrt(mean(s^2) + eps)),  s = out_sum (or x)
+ * rows x H elements, row strides in elements (multiples of 8), H a multiple of 8, H <= 8192.
+ * out_sum may alias x or residual; out_norm may alias x when residual is null. */
+int ksa_add_rmsnorm(const void* x, const void* residual, const void* weight, void* out_norm,
+                    void* out_sum, long long rows, int H, long long x_row_stride,
+                    long long residual_row_stride, long long norm_row_stride,
+                    long long sum_row_stride, int dtype, float eps, void* stream);
+
+/* out = round(SiLU(gate)) * up, the MLP activation of HF:507-514 (act_fn(gate_proj(x)) *
+ * up_proj(x)) in one pass; gate and up may be the two halves of one fused projection output
+ * (row strides in elements, multiples of 8; I a multiple of 8; rows < 2^31). */
+int ksa_silu_mul(const void* gate, const void* up, void* out, long long rows, int I,
+                 long long gate_row_stride, long long up_row_stride, long long out_row_stride,
+                 int dtype, void* stream);
+
 /* Measurement aid (no counterpart in the reference): launches a pure stream of bf16 MFMA
  * 32x32x16 instructions (blocks x waves_per_block waves, 16 * iters instructions each, operands
  * random or all zero) and returns the floating-point operations of the launch in *flop.  Timed

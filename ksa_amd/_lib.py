@@ -30,6 +30,9 @@ _SIGNATURES = {
                        + [ctypes.c_float, _int, _vp, ctypes.c_size_t, _vp]),
     "ksa_copy_rows": (_int, [_vp] * 4 + [_int] * 6 + [_i64p] * 2 + [_vp]),
     "ksa_pre_attention": (_int, [_vp] * 10 + [_int] * 6 + [_i64p] * 7 + [ctypes.c_float, _vp]),
+    "ksa_add_rmsnorm": (_int, [_vp] * 5 + [ctypes.c_longlong, _int] + [ctypes.c_longlong] * 4
+                        + [_int, ctypes.c_float, _vp]),
+    "ksa_silu_mul": (_int, [_vp] * 3 + [ctypes.c_longlong, _int] + [ctypes.c_longlong] * 3 + [_int, _vp]),
     "ksa_probe_mfma_stream": (_int, [_vp] + [_int] * 4 + [ctypes.POINTER(ctypes.c_double), _vp]),
     "ksa_debug_count_visible": (ctypes.c_longlong, [ctypes.c_longlong] * 3 + [_int] * 7),
 }

@@ -1,0 +1,176 @@
+// Two element-wise steps of a decoder layer around the attention path, one pass over HBM each
+// (gfx950), with the rounding points of the reference's 16-bit tensor ops:
+//   * residual add + RMSNorm over the hidden size
+//       examples/pretrain/hf_template/modeling_qwen3sa.py:64-79 (Qwen3RMSNorm.forward: fp32
+//       normalisation, result rounded to the 16-bit type, times the 16-bit weight) and the
+//       residual adds of Qwen3DecoderLayer.forward :946, :952
+//   * SiLU(gate) * up of the MLP (:507-514)
+// Both replace chains of 3-8 library element-wise launches; at decode batch sizes a layer step
+// is bound by the number of launches.
+#include <hip/hip_runtime.h>
+
+#include "ksa_api_internal.h"
+#include "ksa_cvt.h"
+
+namespace {
+
+struct NormParams {
+    const uint16_t* x;
+    const uint16_t* res;   // may be null
+    const uint16_t* w;
+    uint16_t* out_norm;
+    uint16_t* out_sum;     // x + res (null if res is null)
+    int64_t rows;
+    int64_t xs, rs, ns, ss;  // row strides (elements)
+    int H;
+    float eps;
+};
+
+// One wave per row; the row (after the residual add) stays in registers between the
+// sum-of-squares pass and the scaling pass.  NI = 16-byte items per lane.
+template <typename T, int NI>
+__global__ __launch_bounds__(256) void ksa_add_rmsnorm_kernel(const NormParams p) {
+    using C = KsaCvt<T>;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int items = p.H / 8;
+    for (int64_t row = (int64_t)blockIdx.x * 4 + wave; row < p.rows; row += (int64_t)gridDim.x * 4) {
+        u32x4 r[NI];
+        float ss = 0.f;
+#pragma unroll
+        for (int j = 0; j < NI; ++j) {
+            const int idx = lane + 64 * j;
+            if (idx < items) {
+                r[j] = *reinterpret_cast<const u32x4*>(p.x + row * p.xs + 8 * idx);
+                if (p.res) {
+                    const u32x4 q = *reinterpret_cast<const u32x4*>(p.res + row * p.rs + 8 * idx);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        r[j][i] = C::down2(C::lo(r[j][i]) + C::lo(q[i]), C::hi(r[j][i]) + C::hi(q[i]));
+                    *reinterpret_cast<u32x4*>(p.out_sum + row * p.ss + 8 * idx) = r[j];
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float a = C::lo(r[j][i]), b = C::hi(r[j][i]);
+                    ss = fmaf(a, a, ss);
+                    ss = fmaf(b, b, ss);
+                }
+            }
+        }
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1) ss += __shfl_xor(ss, m);
+        const float inv = rsqrtf(ss / (float)p.H + p.eps);
+#pragma unroll
+        for (int j = 0; j < NI; ++j) {
+            const int idx = lane + 64 * j;
+            if (idx < items) {
+                const u32x4 wv = *reinterpret_cast<const u32x4*>(p.w + 8 * idx);
+                u32x4 o;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const uint32_t y = C::down2(C::lo(r[j][i]) * inv, C::hi(r[j][i]) * inv);
+                    o[i] = C::down2(C::lo(wv[i]) * C::lo(y), C::hi(wv[i]) * C::hi(y));
+                }
+                *reinterpret_cast<u32x4*>(p.out_norm + row * p.ns + 8 * idx) = o;
+            }
+        }
+    }
+}
+
+template <typename T, int NI>
+int launch_norm(const NormParams& p, hipStream_t st) {
+    const int64_t blocks = (p.rows + 3) / 4;
+    const int64_t cap = 256 * 32;
+    hipLaunchKernelGGL((ksa_add_rmsnorm_kernel<T, NI>), dim3((unsigned)(blocks < cap ? blocks : cap)), dim3(256), 0,
+                       st, p);
+    return ksa_check_launch();
+}
+
+template <typename T>
+int dispatch_norm(const NormParams& p, hipStream_t st) {
+    const int need = (p.H / 8 + 63) / 64;
+    if (need <= 1) return launch_norm<T, 1>(p, st);
+    if (need <= 2) return launch_norm<T, 2>(p, st);
+    if (need <= 4) return launch_norm<T, 4>(p, st);
+    if (need <= 8) return launch_norm<T, 8>(p, st);
+    if (need <= 16) return launch_norm<T, 16>(p, st);
+    return KSA_ERR_UNSUPPORTED;
+}
+
+struct ActParams {
+    const uint16_t* gate;
+    const uint16_t* up;
+    uint16_t* out;
+    int64_t gs, us, os;  // row strides (elements)
+    int I;
+};
+
+// blockIdx.x = row, blockIdx.y = block of 256 16-byte items inside the row
+template <typename T>
+__global__ __launch_bounds__(256) void ksa_silu_mul_kernel(const ActParams p) {
+    using C = KsaCvt<T>;
+    const int64_t row = blockIdx.x;
+    const int idx = blockIdx.y * 256 + threadIdx.x;
+    if (idx >= p.I / 8) return;
+    const u32x4 g = *reinterpret_cast<const u32x4*>(p.gate + row * p.gs + 8 * idx);
+    const u32x4 u = *reinterpret_cast<const u32x4*>(p.up + row * p.us + 8 * idx);
+    u32x4 o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float a = C::lo(g[i]), b = C::hi(g[i]);
+        const uint32_t s = C::down2(a / (1.f + expf(-a)), b / (1.f + expf(-b)));
+        o[i] = C::down2(C::lo(s) * C::lo(u[i]), C::hi(s) * C::hi(u[i]));
+    }
+    *reinterpret_cast<u32x4*>(p.out + row * p.os + 8 * idx) = o;
+}
+
+bool al16(const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; }
+
+}  // namespace
+
+extern "C" int ksa_add_rmsnorm(const void* x, const void* residual, const void* weight, void* out_norm,
+                               void* out_sum, long long rows, int H, long long x_row_stride,
+                               long long residual_row_stride, long long norm_row_stride,
+                               long long sum_row_stride, int dtype, float eps, void* stream) {
+    if (!x || !weight || !out_norm) return KSA_ERR_NULL;
+    if (residual && !out_sum) return KSA_ERR_NULL;
+    if (rows <= 0 || H <= 0 || H % 8 != 0 || !(eps >= 0.f)) return KSA_ERR_INVALID;
+    if (dtype != KSA_DTYPE_BF16 && dtype != KSA_DTYPE_F16) return KSA_ERR_UNSUPPORTED;
+    if (!al16(x) || !al16(weight) || !al16(out_norm) || (residual && (!al16(residual) || !al16(out_sum))))
+        return KSA_ERR_ALIGN;
+    if (x_row_stride % 8 || norm_row_stride % 8 || (residual && (residual_row_stride % 8 || sum_row_stride % 8)))
+        return KSA_ERR_ALIGN;
+    NormParams p{};
+    p.x = (const uint16_t*)x;
+    p.res = (const uint16_t*)residual;
+    p.w = (const uint16_t*)weight;
+    p.out_norm = (uint16_t*)out_norm;
+    p.out_sum = residual ? (uint16_t*)out_sum : nullptr;
+    p.rows = rows;
+    p.xs = x_row_stride, p.rs = residual_row_stride, p.ns = norm_row_stride, p.ss = sum_row_stride;
+    p.H = H;
+    p.eps = eps;
+    return dtype == KSA_DTYPE_BF16 ? dispatch_norm<KsaBf16>(p, (hipStream_t)stream)
+                                   : dispatch_norm<KsaF16>(p, (hipStream_t)stream);
+}
+
+extern "C" int ksa_silu_mul(const void* gate, const void* up, void* out, long long rows, int I,
+                            long long gate_row_stride, long long up_row_stride, long long out_row_stride,
+                            int dtype, void* stream) {
+    if (!gate || !up || !out) return KSA_ERR_NULL;
+    if (rows <= 0 || rows >= (1ll << 31) || I <= 0 || I % 8 != 0) return KSA_ERR_INVALID;
+    if (dtype != KSA_DTYPE_BF16 && dtype != KSA_DTYPE_F16) return KSA_ERR_UNSUPPORTED;
+    if (!al16(gate) || !al16(up) || !al16(out) || gate_row_stride % 8 || up_row_stride % 8 || out_row_stride % 8)
+        return KSA_ERR_ALIGN;
+    const int yblocks = (I / 8 + 255) / 256;
+    if (yblocks > 65535) return KSA_ERR_INVALID;
+    ActParams p{(const uint16_t*)gate, (const uint16_t*)up, (uint16_t*)out, gate_row_stride, up_row_stride,
+                out_row_stride, I};
+    if (dtype == KSA_DTYPE_BF16)
+        hipLaunchKernelGGL(ksa_silu_mul_kernel<KsaBf16>, dim3((unsigned)rows, yblocks), dim3(256), 0,
+                           (hipStream_t)stream, p);
+    else
+        hipLaunchKernelGGL(ksa_silu_mul_kernel<KsaF16>, dim3((unsigned)rows, yblocks), dim3(256), 0,
+                           (hipStream_t)stream, p);
+    return ksa_check_launch();
+}

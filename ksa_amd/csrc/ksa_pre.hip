@@ -20,6 +20,7 @@
 
 #include "ksa_api_internal.h"
 #include "ksa_tile.h"
+#include "ksa_cvt.h"
 
 namespace {
 
@@ -37,40 +38,7 @@ struct PreParams {
 };
 
 template <typename T>
-struct PreCvt;
-template <>
-struct PreCvt<KsaBf16> {
-    static __device__ __forceinline__ float up(uint16_t u) {
-        return __builtin_bit_cast(float, (uint32_t)u << 16);
-    }
-    static __device__ __forceinline__ uint16_t down(float f) {
-        return __builtin_bit_cast(uint16_t, (__bf16)f);
-    }
-    // two values rounded into one word (low, high) and back
-    static __device__ __forceinline__ uint32_t down2(float lo, float hi) { return KsaOps<KsaBf16>::pack2(lo, hi); }
-    static __device__ __forceinline__ float lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
-    static __device__ __forceinline__ float hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
-};
-template <>
-struct PreCvt<KsaF16> {
-    // Conversion instructions written out: with plain _Float16 casts the compiler may keep
-    // excess precision across a down/up pair, which would drop the rounding points.
-    static __device__ __forceinline__ float up(uint16_t u) {
-        float f;
-        asm("v_cvt_f32_f16 %0, %1" : "=v"(f) : "v"((uint32_t)u));
-        return f;
-    }
-    static __device__ __forceinline__ uint16_t down(float f) {
-        uint32_t h;
-        asm("v_cvt_f16_f32 %0, %1" : "=v"(h) : "v"(f));
-        return (uint16_t)h;
-    }
-    static __device__ __forceinline__ uint32_t down2(float lo, float hi) {
-        return (uint32_t)down(lo) | ((uint32_t)down(hi) << 16);
-    }
-    static __device__ __forceinline__ float lo(uint32_t w) { return up((uint16_t)(w & 0xffffu)); }
-    static __device__ __forceinline__ float hi(uint32_t w) { return up((uint16_t)(w >> 16)); }
-};
+using PreCvt = KsaCvt<T>;
 
 // value of the lane `n` places further inside the same row of 16 lanes (cyclic)
 template <int N>

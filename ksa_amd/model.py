@@ -13,16 +13,17 @@ token, plus the summary tokens when the chunk completes, and their position ids)
 Differences from the reference, on purpose:
 * any batch size (the reference refuses batch > 1 at :753; its cache tensors and counters are
   already batch-shaped, all sequences of a batch have the same length);
-* weights are plain tensors (fused q|k|v and gate|up matrices), not nn.Modules; projections and
-  the MLP are torch matmuls (hipBLASLt), everything attention-side is this package's kernels;
+* weights are plain tensors (fused q|k|v and gate|up matrices), not nn.Modules; the GEMMs are
+  torch matmuls (hipBLASLt), everything else (pre-attention, attention, cache rows, residual add +
+  RMSNorm, SiLU-mul) is this package's kernels;
 * a "full attention" layer is, as in the reference's inference model, a Summary layer whose
   window is larger than any sequence (append-only text cache, :114-115, :232-242);
 * `summary_independent_parameters` is supported for mix_coeff 0 and 1 (the reference's default
   1.0, :765-791): the summary rows then take their q, k, v from their own projection.
 
-The attention-side operators come from an `ops` object; the default binds the HIP kernels of this
-package and needs a GPU.  Tests pass a CPU fp32 implementation of the same four operators to
-obtain the reference run of this very module.
+The attention-side and element-wise operators come from an `ops` object; the default binds the
+HIP kernels of this package and needs a GPU.  Tests pass a CPU fp32 implementation of the same
+operators to obtain the reference run of this very module.
 """
 from __future__ import annotations
 
@@ -127,10 +128,12 @@ class HipOps:
     """The attention-side operators of the model, bound to this package's HIP kernels."""
 
     def __init__(self):
-        from . import cache, decode, pre, prefill
+        from . import cache, decode, elementwise, pre, prefill
         self.cache_cls = cache.Qwen3RingBufferCache
         self.pre_attention = pre.pre_attention
         self.summary_attn_func = prefill.summary_attn_func
+        self.add_rmsnorm = elementwise.add_rmsnorm
+        self.silu_mul = elementwise.silu_mul
         self._decode = decode.ksa_decode
 
     def decode(self, q, kbuf, vbuf, start, end, scale):
@@ -216,10 +219,11 @@ class KsaQwen3ForCausalLM:
         self.lm_head = emb[: config.vocab_size] if config.tie_word_embeddings else weights["lm_head"]
 
     # ---- pieces ----------------------------------------------------------------------
-    def _rms(self, x, w):
-        xf = x.float()
-        xf = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + self.config.rms_norm_eps)
-        return w * xf.to(x.dtype)
+    def _add_norm(self, delta, x, w):
+        """(x + delta, w * rmsnorm(x + delta)); delta None: (x, w * rmsnorm(x))."""
+        if delta is None:
+            return self.ops.add_rmsnorm(x, None, w, self.config.rms_norm_eps)
+        return self.ops.add_rmsnorm(delta, x, w, self.config.rms_norm_eps)
 
     def _rope_tables(self, position_ids):
         """cos, sin [1, L, D] in the model dtype from position ids [1, L] (computed in fp32)."""
@@ -244,10 +248,11 @@ class KsaQwen3ForCausalLM:
     def _mlp(self, lw, x):
         gu = F.linear(x, lw["gate_up_proj"])
         I = self.config.intermediate_size
-        return F.linear(F.silu(gu[..., :I]) * gu[..., I:], lw["down_proj"])
+        return F.linear(self.ops.silu_mul(gu[..., :I], gu[..., I:]), lw["down_proj"])
 
-    def _logits(self, hidden_last):
-        return F.linear(self._rms(hidden_last, self.w["norm"]), self.lm_head)
+    def _logits(self, x_last, delta_last):
+        _, h = self._add_norm(delta_last, x_last, self.w["norm"])
+        return F.linear(h, self.lm_head)[..., : self.config.vocab_size]
 
     # ---- prefill ---------------------------------------------------------------------
     @torch.no_grad()
@@ -262,19 +267,20 @@ class KsaQwen3ForCausalLM:
         cos, sin = self._rope_tables(pos)
         cache = ops.cache_cls(cfg, self.scns)
         x = self.w["embed_tokens"][ids]
+        delta = None     # output of the previous MLP, added to the residual stream by the next norm
         Hkv, D = cfg.num_key_value_heads, cfg.head_dim
         for li, lw in enumerate(self.w["layers"]):
-            h = self._rms(x, lw["input_layernorm"])
+            x, h = self._add_norm(delta, x, lw["input_layernorm"])
             q, k, v = self._qkv(lw, h, sum_rows)
             k_slot, v_slot = cache.prefill_slots(li, b, Hkv, L, D, self.dtype, self.device, n_sum)
             q, k, v = ops.pre_attention(q, k, v, lw["q_norm"], lw["k_norm"], cos, sin, cfg.rms_norm_eps,
                                         k_out=k_slot, v_out=v_slot)
             attn, _ = ops.summary_attn_func(q, k, v, C, S, self.scns[li], summary_pos=is_sum)
-            x = x + F.linear(attn.reshape(b, L, -1), lw["o_proj"])
-            x = x + self._mlp(lw, self._rms(x, lw["post_attention_layernorm"]))
+            x, h = self._add_norm(F.linear(attn.reshape(b, L, -1), lw["o_proj"]), x, lw["post_attention_layernorm"])
+            delta = self._mlp(lw, h)
         cache.reorganize_after_prefill(is_sum[None])
         last_text = L - 1 if (L % (C + S)) != 0 else L - 1 - S   # the last prompt token's slot
-        return self._logits(x[:, last_text:last_text + 1])[..., : cfg.vocab_size], cache
+        return self._logits(x[:, last_text:last_text + 1], delta[:, last_text:last_text + 1]), cache
 
     # ---- decode ----------------------------------------------------------------------
     @torch.no_grad()
@@ -299,8 +305,9 @@ class KsaQwen3ForCausalLM:
             sum_rows = None
         cos, sin = self._rope_tables(pos)
         x = self.w["embed_tokens"][ids]
+        delta = None
         for li, lw in enumerate(self.w["layers"]):
-            h = self._rms(x, lw["input_layernorm"])
+            x, h = self._add_norm(delta, x, lw["input_layernorm"])
             q, k, v = self._qkv(lw, h, sum_rows)
             if not boundary:
                 k_slot, v_slot = cache.text_slots(li, b, Hkv, D, self.dtype, self.device)
@@ -320,10 +327,11 @@ class KsaQwen3ForCausalLM:
                 sum_out = ops.decode(qh[:, :, 1:], k_cs, v_cs, 0, k_cs.shape[2], self.scaling)
                 cache.update_summary(kh[:, :, 1:], vh[:, :, 1:], li)
                 attn = torch.cat([text_out, sum_out], dim=1)
-            x = x + F.linear(attn.reshape(b, ids.shape[1], -1), lw["o_proj"])
-            x = x + self._mlp(lw, self._rms(x, lw["post_attention_layernorm"]))
+            x, h = self._add_norm(F.linear(attn.reshape(b, ids.shape[1], -1), lw["o_proj"]), x,
+                                  lw["post_attention_layernorm"])
+            delta = self._mlp(lw, h)
         cache.reset_chunk_counter()
-        return self._logits(x[:, :1])[..., : cfg.vocab_size]
+        return self._logits(x[:, :1], delta[:, :1])
 
     # ---- driver ----------------------------------------------------------------------
     def forward(self, input_ids: torch.Tensor, cache=None):

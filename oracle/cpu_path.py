@@ -80,3 +80,18 @@ def pre_attention(q, k, v, q_weight, k_weight, cos, sin, eps=1e-6):
     s = sin.unsqueeze(2)
     qn, kn = rms(q, q_weight), rms(k, k_weight)
     return qn * c + rot(qn) * s, kn * c + rot(kn) * s, v
+
+
+def add_rmsnorm(x, residual, weight, eps=1e-6):
+    """Residual add followed by Qwen3RMSNorm.forward, with torch CPU tensor ops in the input
+    dtype (examples/pretrain/hf_template/modeling_qwen3sa.py:64-79 and the adds at :946, :952).
+    Returns (x + residual, weight * norm(x + residual))."""
+    s = x if residual is None else x + residual
+    sf = s.to(torch.float32)
+    sf = sf * torch.rsqrt(sf.pow(2).mean(-1, keepdim=True) + eps)
+    return s, weight * sf.to(s.dtype)
+
+
+def silu_mul(gate, up):
+    """act_fn(gate) * up of Qwen3MLP.forward (:507-514) in the input dtype."""
+    return F.silu(gate) * up

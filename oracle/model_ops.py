@@ -1,4 +1,4 @@
-"""CPU fp32 stand-ins for the four attention-side operators of `ksa_amd.model`, built from
+"""CPU fp32 stand-ins for the attention-side and element-wise operators of `ksa_amd.model`, built from
 the oracle's restatements.  TEST INFRASTRUCTURE ONLY: with these the build's own end-to-end
 module runs on the host in fp32, which is the run its GPU results are compared with.
 
@@ -6,7 +6,8 @@ Follows examples/pretrain/hf_template/modeling_qwen3sa.py: :64-79, :516-554, :66
 (pre-attention, via cpu_path.pre_attention), whl-sa summary_attn/interface.py:271-289 (the
 summary rows form the key prefix; dense masked soft-max via ksa_oracle.masked_attention),
 :557-566, :591-612 (decode: un-masked soft-max over the cache slice), :85-505 (the cache,
-product bookkeeping with a host row mover).
+product bookkeeping with a host row mover), :64-79, :507-514, :946, :952 (residual add + RMSNorm,
+SiLU-mul, via cpu_path).
 """
 from __future__ import annotations
 
@@ -42,6 +43,9 @@ class OracleOps:
                 val = given
             res.append(val)
         return tuple(res)
+
+    add_rmsnorm = staticmethod(cpu_path.add_rmsnorm)
+    silu_mul = staticmethod(cpu_path.silu_mul)
 
     @staticmethod
     def summary_attn_func(q, k, v, C, S, W, summary_pos=None):
