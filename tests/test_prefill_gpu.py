@@ -222,6 +222,60 @@ def test_prefill_cfg1_sampled_rows(wave_rows):
     assert np.abs(lse[:, rows] - wlse).max() <= 2e-3
 
 
+def test_prefill_cfg2_sampled_rows():
+    """cfg 2 (128k text tokens, 1024 chunks, 32/8 heads), the benchmark's shape: every row of the
+    first and last two chunks, offsets {0, C-1, C, B-1} of 32 random chunks and 256 random rows
+    against the oracle."""
+    Sq, Hq, Hkv, D, C, S, W = 139264, 32, 8, 128, 128, 8, 4
+    q, k, v = make_qkv(Sq, Hq, Hkv, D, seed=0)
+    sp = O.summary_positions(Sq, C, S)
+    got, lse = _run_prefill(q, k, v, C, S, W, sp)
+    rng = np.random.default_rng(2)
+    B = C + S
+    rows = set(range(0, 2 * B)) | set(range(Sq - 2 * B, Sq))
+    for c in rng.choice(Sq // B, 32, replace=False):
+        rows |= {c * B, c * B + C - 1, c * B + C, c * B + B - 1}
+    rows |= set(rng.choice(Sq, 256, replace=False).tolist())
+    rows = np.array(sorted(rows), np.int32)
+    want, wlse = c_oracle.attention_rows(to_np(q), to_np(k), to_np(v), C, S, W, summary_pos=sp, rows=rows)
+    _compare(got[rows], want, "cfg2 sampled rows")
+    assert np.abs(lse[:, rows] - wlse).max() <= 2e-3
+
+
+def test_prefill_cfg2_visibility_probe_all_rows():
+    """Every row of the 128k shape: with Q = K = 0 and V = one-hot of (position mod 128) the
+    output is count-of-class / n_i over the row's visible set.  All probabilities are exactly 1,
+    so the only error is the final rounding to bf16 and one wrongly (un)masked key moves a value
+    by about 1 / 69 of itself.  Expected counts come from the interval form of the rule (text:
+    summaries of chunks < c - W, text of chunks c - W .. c - 1, own chunk causally; summary: own
+    chunk's text and its summaries causally), by prefix sums over positions."""
+    Sq, Hq, Hkv, D, C, S, W = 139264, 2, 1, 128, 128, 8, 4
+    B = C + S
+    pos = np.arange(Sq)
+    is_sum = (pos % B) >= C
+    cls = pos % D
+    onehot = np.zeros((Sq, D), np.int32)
+    onehot[pos, cls] = 1
+    cumT = np.concatenate([np.zeros((1, D), np.int32), np.cumsum(onehot * (~is_sum)[:, None], axis=0, dtype=np.int32)])
+    cumS = np.concatenate([np.zeros((1, D), np.int32), np.cumsum(onehot * is_sum[:, None], axis=0, dtype=np.int32)])
+    c = pos // B
+    lo = np.maximum(c - W, 0) * B                       # first in-line position of the window
+    text_rows = cumS[lo] + (cumT[pos + 1] - cumT[lo])
+    sum_rows = (cumT[c * B + C] - cumT[c * B]) + (cumS[pos + 1] - cumS[c * B])
+    cnt = np.where(is_sum[:, None], sum_rows, text_rows).astype(np.float64)
+    want = cnt / cnt.sum(axis=1, keepdims=True)
+    q = torch.zeros(Sq, Hq, D, dtype=torch.bfloat16)
+    k = torch.zeros(Sq, Hkv, D, dtype=torch.bfloat16)
+    v = torch.zeros(Sq, Hkv, D, dtype=torch.bfloat16)
+    v[torch.arange(Sq), 0, torch.from_numpy(cls)] = 1.0
+    got, lse = _run_prefill(q, k, v, C, S, W, O.summary_positions(Sq, C, S))
+    for h in range(Hq):
+        err = np.abs(got[:, h] - want)
+        assert (err <= want * 2.0 ** -8 + 1e-7).all(), (h, float(err.max()))
+    # lse = log(n_i) since every score is 0
+    assert np.abs(lse - np.log(cnt.sum(axis=1))[None, :]).max() <= 1e-4
+
+
 def test_prefill_batch_and_fp16(wave_rows):
     Sq, Hq, Hkv, D, C, S, W = 680, 4, 2, 128, 128, 8, 1
     import ksa_amd
