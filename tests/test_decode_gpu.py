@@ -99,6 +99,37 @@ def test_decode_cfg3_shape_subset():
     _check(q, k, v, 136 - cbl, np.full(Bz, 8808, np.int32), None)
 
 
+def test_decode_cfg3_full_batch():
+    """cfg 3 itself: batch 64, 32/8 heads, cap 17288, per-sequence slice [136 - cbl, 8808) with
+    cbl uniform in [1, 128]: all 64 x 32 output rows against the oracle (one sequence at a
+    time on the host), and the split-K identity (1 split == 4 splits up to rounding)."""
+    import ksa_amd
+    dev = torch.device("cuda")
+    Bz, Hq, Hkv, D, cap = 64, 32, 8, 128, 17288
+    g = torch.Generator(device=dev).manual_seed(11)
+    k = torch.randn(Bz, Hkv, cap, D, generator=g, device=dev).to(torch.bfloat16)
+    v = torch.randn(Bz, Hkv, cap, D, generator=g, device=dev).to(torch.bfloat16)
+    q = torch.randn(Bz, Hq, 1, D, generator=g, device=dev).to(torch.bfloat16)
+    cbl = torch.randint(1, 129, (Bz,), generator=g, device=dev, dtype=torch.int32)
+    start = (136 - cbl).to(torch.int32)
+    end = torch.full((Bz,), 8808, dtype=torch.int32, device=dev)
+    out1 = ksa_amd.ksa_decode(q, k, v, start, end, nsplit=1)
+    out4 = ksa_amd.ksa_decode(q, k, v, start, end, nsplit=4)
+    outa = ksa_amd.ksa_decode(q, k, v, start, end)
+    torch.cuda.synchronize()
+    assert (out1.float() - out4.float()).abs().max().item() <= 2e-3
+    assert (out1.float() - outa.float()).abs().max().item() <= 2e-3
+    got = to_np(out1)
+    st, en = start.cpu().numpy(), end.cpu().numpy()
+    worst = 0.0
+    for b in range(Bz):
+        want = c_oracle.decode(to_np(q[b:b + 1]), to_np(k[b:b + 1]), to_np(v[b:b + 1]), st[b:b + 1], en[b:b + 1])
+        err = np.abs(got[b:b + 1] - want).max()
+        worst = max(worst, err)
+        assert err <= ATOL and err <= RTOL_INF * np.abs(want).max(), (b, err)
+    assert np.isfinite(got).all()
+
+
 def test_copy_rows():
     import ksa_amd
     from ksa_amd.cache import _move_rows
