@@ -20,6 +20,11 @@ struct KsaCvt<KsaBf16> {
     static __device__ __forceinline__ uint32_t down2(float lo, float hi) { return KsaOps<KsaBf16>::pack2(lo, hi); }
     static __device__ __forceinline__ float lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
     static __device__ __forceinline__ float hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
+    // a.lo * b.lo + a.hi * b.hi + c on packed pairs (the products of two 16-bit values are exact in fp32)
+    static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), c, false);
+    }
+    static constexpr uint32_t kOnes = 0x3f803f80u;  // (1.0, 1.0)
 };
 template <>
 struct KsaCvt<KsaF16> {
@@ -32,7 +37,9 @@ struct KsaCvt<KsaF16> {
     }
     static __device__ __forceinline__ uint16_t down(float f) {
         uint32_t h;
-        asm("v_cvt_f16_f32 %0, %1" : "=v"(h) : "v"(f));
+        // the wait states cover a packed-dot-product result as the input: the compiler's hazard
+        // handling does not look inside an assembly statement (3 wait states, DOT -> VALU)
+        asm("s_nop 2\n\tv_cvt_f16_f32 %0, %1" : "=v"(h) : "v"(f));
         return (uint16_t)h;
     }
     static __device__ __forceinline__ uint32_t down2(float lo, float hi) {
@@ -40,5 +47,9 @@ struct KsaCvt<KsaF16> {
     }
     static __device__ __forceinline__ float lo(uint32_t w) { return up((uint16_t)(w & 0xffffu)); }
     static __device__ __forceinline__ float hi(uint32_t w) { return up((uint16_t)(w >> 16)); }
+    static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a), __builtin_bit_cast(f16x2, b), c, false);
+    }
+    static constexpr uint32_t kOnes = 0x3c003c00u;
 };
 

@@ -34,6 +34,7 @@ struct PreParams {
     int64_t d_bs[3], d_rs[3], d_hs[3];
     int64_t c_bs, c_rs;
     int batch, S, Hq, Hkv;
+    int tok_per_pass;  // tokens per workgroup pass: 4 / gcd(row groups per token, 4)
     float eps;
 };
 
@@ -61,11 +62,14 @@ __device__ __forceinline__ float pre_row_sum(float ss) {
     return ss;
 }
 
-// One workgroup takes one token at a time (grid-stride over tokens); its four waves share
-// the token's head rows, RPW rows of one of q / k / v per wave instruction.  Which tensor a
-// wave instruction works on, the token's base addresses and the weights are wave-uniform
-// (scalar registers); a lane only adds its row's offset, so no index division or 64-bit
-// multiply sits in the inner loop, and cos / sin are fetched once per wave and token.
+// One workgroup takes a few consecutive tokens at a time (grid-stride); its four waves share
+// their head rows, RPW rows of one of q / k / v per wave instruction, the same number for every
+// wave.  Which tensor a wave instruction works on, the token's base addresses and the weights
+// are wave-uniform (scalar registers); a lane only adds its row's offset, so no index division
+// or 64-bit multiply sits in the inner loop.  Products of two 16-bit values are taken with
+// packed dot products against operands that hold one element and a zero, straight from the
+// packed words (exact in fp32), and the final sum of the two rounded terms is a dot product
+// with (1, 1).
 template <typename T, int D>
 __global__ __launch_bounds__(256) void ksa_pre_attention_kernel(const PreParams p) {
     using C = PreCvt<T>;
@@ -82,16 +86,19 @@ __global__ __launch_bounds__(256) void ksa_pre_attention_kernel(const PreParams 
     // rotate_half: the first half of a row takes -z[j + D/2], the second half +z[j - D/2];
     // the sign goes into the sine once per token
     const uint32_t sgn_bits = t < LPR / 2 ? 0x80008000u : 0u;
-    float wqf[8], wkf[8];  // this lane's slice of the two weight vectors
+    // this lane's slice of the two weight vectors, each packed word split into (low, 0) and
+    // (0, high): a packed dot product with such a word is the exact fp32 product of one element,
+    // taken straight from packed operands
+    uint32_t wlo[2][4], whi[2][4];
     {
         const u32x4 wq = *reinterpret_cast<const u32x4*>(p.w[0] + 8 * t);
         const u32x4 wk = *reinterpret_cast<const u32x4*>(p.w[1] + 8 * t);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            wqf[2 * i] = C::lo(wq[i]);
-            wqf[2 * i + 1] = C::hi(wq[i]);
-            wkf[2 * i] = C::lo(wk[i]);
-            wkf[2 * i + 1] = C::hi(wk[i]);
+            wlo[0][i] = wq[i] & 0xffffu;
+            whi[0][i] = wq[i] & 0xffff0000u;
+            wlo[1][i] = wk[i] & 0xffffu;
+            whi[1][i] = wk[i] & 0xffff0000u;
         }
     }
     // element offset of this lane's row inside a wave instruction's block of rows
@@ -102,20 +109,36 @@ __global__ __launch_bounds__(256) void ksa_pre_attention_kernel(const PreParams 
         ldst[w] = (uint32_t)sub * (uint32_t)p.d_hs[w] + 8 * t;
     }
 
-    for (int tok = blockIdx.x; tok < ntok; tok += gridDim.x) {
-        const int b = tok / p.S;
-        const int s = tok - b * p.S;
-        const u32x4 craw = *reinterpret_cast<const u32x4*>(p.cos + b * p.c_bs + (int64_t)s * p.c_rs + 8 * t);
-        const u32x4 sraw = *reinterpret_cast<const u32x4*>(p.sin + b * p.c_bs + (int64_t)s * p.c_rs + 8 * t);
-        float cs[8], sn[8];  // unpacked once per token; the sine carries the rotate_half sign
+    // A workgroup pass covers TOK consecutive tokens, TOK * G row groups in all, a multiple of
+    // four, so that its four waves get the same number of groups (G = 6 with 32 + 8 + 8 heads of
+    // 128: two tokens, three groups per wave).  (token, group) advance by four per wave step.
+    const int TOK = p.tok_per_pass;
+    const int gi0 = wave % G, tl0 = wave / G;
+    for (int t0 = blockIdx.x * TOK; t0 < ntok; t0 += gridDim.x * TOK) {
+        int cur = -1;
+        uint32_t clo[4], chi[4], slo[4], shi[4];
+        int b = 0, s = 0;
+        for (int gi = gi0, tl = tl0; tl < TOK; gi += 4) {
+            while (gi >= G) {
+                gi -= G;
+                ++tl;
+            }
+            const int tok = t0 + tl;
+            if (tl >= TOK || tok >= ntok) break;
+            if (tok != cur) {  // wave-uniform: the rotary row of this token, split like the weights
+                cur = tok;
+                b = tok / p.S;
+                s = tok - b * p.S;
+                const u32x4 craw = *reinterpret_cast<const u32x4*>(p.cos + b * p.c_bs + (int64_t)s * p.c_rs + 8 * t);
+                const u32x4 sraw = *reinterpret_cast<const u32x4*>(p.sin + b * p.c_bs + (int64_t)s * p.c_rs + 8 * t);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            cs[2 * i] = C::lo(craw[i]);
-            cs[2 * i + 1] = C::hi(craw[i]);
-            sn[2 * i] = C::lo(sraw[i] ^ sgn_bits);
-            sn[2 * i + 1] = C::hi(sraw[i] ^ sgn_bits);
-        }
-        for (int gi = wave; gi < G; gi += 4) {
+                for (int i = 0; i < 4; ++i) {  // the sine carries the rotate_half sign
+                    clo[i] = craw[i] & 0xffffu;
+                    chi[i] = craw[i] & 0xffff0000u;
+                    slo[i] = (sraw[i] ^ sgn_bits) & 0xffffu;
+                    shi[i] = (sraw[i] ^ sgn_bits) & 0xffff0000u;
+                }
+            }
             const int which = gi < Gq ? 0 : (gi < Gq + Gk ? 1 : 2);          // wave-uniform
             const int h0 = (gi - (which == 0 ? 0 : (which == 1 ? Gq : Gq + Gk))) * RPW;
             const uint16_t* sbase = p.src[which] + b * p.s_bs[which] + (int64_t)s * p.s_rs[which] + (int64_t)h0 * p.s_hs[which];
@@ -127,35 +150,33 @@ __global__ __launch_bounds__(256) void ksa_pre_attention_kernel(const PreParams 
                 *reinterpret_cast<u32x4*>(dp) = raw;
                 continue;
             }
-            float x[8];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                x[2 * i] = C::lo(raw[i]);
-                x[2 * i + 1] = C::hi(raw[i]);
-            }
             float ss = 0.f;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) ss = fmaf(x[i], x[i], ss);
+            for (int i = 0; i < 4; ++i) ss = C::dot2(raw[i], raw[i], ss);
             ss = pre_row_sum<LPR>(ss);
             const float inv = rsqrtf(ss * (1.0f / D) + p.eps);
             // z = round(w * round(x * inv)), kept packed for the exchange
             u32x4 zp;
+            auto scale_rows = [&](const uint32_t (&wl)[4], const uint32_t (&wh)[4]) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const uint32_t y = C::down2(x[2 * i] * inv, x[2 * i + 1] * inv);
-                const float w0 = which == 0 ? wqf[2 * i] : wkf[2 * i];
-                const float w1 = which == 0 ? wqf[2 * i + 1] : wkf[2 * i + 1];
-                zp[i] = C::down2(w0 * C::lo(y), w1 * C::hi(y));
-            }
+                for (int i = 0; i < 4; ++i) {
+                    const uint32_t y = C::down2(C::lo(raw[i]) * inv, C::hi(raw[i]) * inv);
+                    zp[i] = C::down2(C::dot2(y, wl[i], 0.f), C::dot2(y, wh[i], 0.f));
+                }
+            };
+            if (which == 0) scale_rows(wlo[0], whi[0]);
+            else scale_rows(wlo[1], whi[1]);
+            // out = round(round(z cos) + round(rot(z) sin)); the two rounded terms of an element
+            // are packed together and added by a dot product with (1, 1)
             u32x4 outp;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 uint32_t pp;  // the partner half of the row
                 if constexpr (LPR == 16) pp = pre_row_ror<8>(zp[i]);
                 else pp = (uint32_t)__shfl_xor((int)zp[i], LPR / 2);
-                const uint32_t zc = C::down2(C::lo(zp[i]) * cs[2 * i], C::hi(zp[i]) * cs[2 * i + 1]);
-                const uint32_t rs = C::down2(C::lo(pp) * sn[2 * i], C::hi(pp) * sn[2 * i + 1]);
-                outp[i] = C::down2(C::lo(zc) + C::lo(rs), C::hi(zc) + C::hi(rs));
+                const uint32_t e0 = C::down2(C::dot2(zp[i], clo[i], 0.f), C::dot2(pp, slo[i], 0.f));
+                const uint32_t e1 = C::down2(C::dot2(zp[i], chi[i], 0.f), C::dot2(pp, shi[i], 0.f));
+                outp[i] = C::down2(C::dot2(e0, C::kOnes, 0.f), C::dot2(e1, C::kOnes, 0.f));
             }
             *reinterpret_cast<u32x4*>(dp) = outp;
         }
@@ -163,8 +184,11 @@ __global__ __launch_bounds__(256) void ksa_pre_attention_kernel(const PreParams 
 }
 
 template <typename T, int D>
-int launch_pre(const PreParams& p, hipStream_t stream) {
-    int64_t blocks = (int64_t)p.batch * p.S;             // one token per workgroup pass
+int launch_pre(PreParams p, hipStream_t stream) {
+    constexpr int RPW = 64 / (D / 8);
+    const int G = (p.Hq + RPW - 1) / RPW + 2 * ((p.Hkv + RPW - 1) / RPW);
+    p.tok_per_pass = (G % 4 == 0) ? 1 : (G % 2 == 0 ? 2 : 4);
+    int64_t blocks = ((int64_t)p.batch * p.S + p.tok_per_pass - 1) / p.tok_per_pass;
     const int64_t cap = 256 * 16;                        // grid-stride beyond that
     if (blocks > cap) blocks = cap;
     hipLaunchKernelGGL((ksa_pre_attention_kernel<T, D>), dim3((unsigned)blocks), dim3(256), 0, stream, p);
