@@ -6,7 +6,7 @@ oracle function is fixed by checks that a plausible mistake would fail:
                            j <-> in-line row (j//S)*B + C + j%S), closed-form row counts,
                            special cases (W >= chunks = causal over text, W = 0, row sees itself)
   block index              known totals for cfg 0 / cfg 1 derived independently (by hand from
-                           the rule, recorded in BASELINE.md), format invariants, C vs numpy
+                           the rule), format invariants, C vs numpy
   masked attention         torch SDPA with an explicit bool mask (library routine), un-masked
                            and plain-causal special cases, numpy vs C implementations
   decode attention         torch SDPA; partition identity of the split merge
