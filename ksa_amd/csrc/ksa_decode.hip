@@ -109,14 +109,18 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_decode_kernel(const DecodePar
     u32x4 kreg[KLD];
     u32x4 vreg[KLD];
 
+    // K/V rows are read once and never again: non-temporal loads
+    auto load_piece = [&](int row0, int i) {
+        const int u = lane + 64 * i;
+        const int row = min(row0 + u / CPR, last_row);
+        kreg[i] = __builtin_nontemporal_load(
+            reinterpret_cast<const u32x4*>(kbase + (int64_t)row * p.k_rs + 8 * (u % CPR)));
+        vreg[i] = __builtin_nontemporal_load(
+            reinterpret_cast<const u32x4*>(vbase + (int64_t)row * p.v_rs + 8 * (u % CPR)));
+    };
     auto load_tile = [&](int row0) {
 #pragma unroll
-        for (int i = 0; i < KLD; ++i) {
-            const int u = lane + 64 * i;
-            const int row = min(row0 + u / CPR, last_row);
-            kreg[i] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)row * p.k_rs + 8 * (u % CPR));
-            vreg[i] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)row * p.v_rs + 8 * (u % CPR));
-        }
+        for (int i = 0; i < KLD; ++i) load_piece(row0, i);
     };
 
     floatx16 oacc[DB];
@@ -133,15 +137,18 @@ __global__ __launch_bounds__(kThreads, 2) void ksa_decode_kernel(const DecodePar
 
     for (; row0 < s1; row0 += kWaves * kRows) {
         ksa_wave_lds_fence();
+        // registers -> LDS, and each register pair is refilled with the next tile right behind
+        // its store, so the loads of the next tile are in flight for the whole step
+        const int next = row0 + kWaves * kRows;
+        const bool has_next = next < s1;
 #pragma unroll
         for (int i = 0; i < KLD; ++i) {
             const int u = lane + 64 * i;
             *reinterpret_cast<u32x4*>(Kw + (u / CPR) * KROW + 8 * (u % CPR)) = kreg[i];
             *reinterpret_cast<u32x4*>(Vw + (u / CPR) * VROW + 8 * (u % CPR)) = vreg[i];
+            if (has_next) load_piece(next, i);
         }
         ksa_wave_lds_fence();
-        const int next = row0 + kWaves * kRows;
-        if (next < s1) load_tile(next);
 
         floatx16 sacc;
 #pragma unroll

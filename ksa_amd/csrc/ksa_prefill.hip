@@ -496,21 +496,6 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
             if (vt >= 1 && vt - 1 < NCH) stage_b(vt - 1);
             if (vt < NCH) stage_a(vt);
         };
-        auto prob2 = [&](int cc) {
-            stage_a(cc);
-            stage_b(cc);
-            stage_c(cc);
-            stage_d(cc);
-        };
-        auto probabilities = [&]() {
-#pragma unroll
-            for (int r = 0; r < RB; ++r) {
-                mc[r] = row_vis[r] ? m_ref[r] * c2 : INFINITY;
-                l_tile[r] = 0.f;
-            }
-#pragma unroll
-            for (int cc = 0; cc < 16 * RB; ++cc) prob2(cc);
-        };
         // move the reference of the rows whose maximum outgrew it (or that have none yet)
         auto rebase = [&]() {
 #pragma unroll
