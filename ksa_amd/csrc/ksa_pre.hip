@@ -144,10 +144,11 @@ __global__ __launch_bounds__(256) void ksa_pre_attention_kernel(const PreParams 
             const uint16_t* sbase = p.src[which] + b * p.s_bs[which] + (int64_t)s * p.s_rs[which] + (int64_t)h0 * p.s_hs[which];
             uint16_t* dbase = p.dst[which] + b * p.d_bs[which] + (int64_t)s * p.d_rs[which] + (int64_t)h0 * p.d_hs[which];
             if (h0 + sub >= Hn[which]) continue;  // a whole lane group is idle: its exchange partners are idle too
-            const u32x4 raw = *reinterpret_cast<const u32x4*>(sbase + lsrc[which]);
+            // every byte is touched once: non-temporal accesses
+            const u32x4 raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(sbase + lsrc[which]));
             uint16_t* dp = dbase + ldst[which];
             if (which == 2) {  // v: layout change only
-                *reinterpret_cast<u32x4*>(dp) = raw;
+                __builtin_nontemporal_store(raw, reinterpret_cast<u32x4*>(dp));
                 continue;
             }
             float ss = 0.f;
@@ -178,7 +179,7 @@ __global__ __launch_bounds__(256) void ksa_pre_attention_kernel(const PreParams 
                 const uint32_t e1 = C::down2(C::dot2(zp[i], chi[i], 0.f), C::dot2(pp, shi[i], 0.f));
                 outp[i] = C::down2(C::dot2(e0, C::kOnes, 0.f), C::dot2(e1, C::kOnes, 0.f));
             }
-            *reinterpret_cast<u32x4*>(dp) = outp;
+            __builtin_nontemporal_store(outp, reinterpret_cast<u32x4*>(dp));
         }
     }
 }
