@@ -37,7 +37,7 @@ __global__ __launch_bounds__(256) void ksa_copy_rows_kernel(const CopyParams p) 
         const int i = (int)(u / p.cpr), c = (int)(u % p.cpr);
         const int sr = p.src_index ? p.src_index[i] : p.src_start + i;
         *reinterpret_cast<u32x4*>(db + (int64_t)(d0 + i) * p.d_rs + 8 * c) =
-            *reinterpret_cast<const u32x4*>(sb + (int64_t)sr * p.s_rs + 8 * c);
+            __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(sb + (int64_t)sr * p.s_rs + 8 * c));
     }
 }
 

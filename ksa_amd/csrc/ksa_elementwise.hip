@@ -27,7 +27,8 @@ struct NormParams {
 };
 
 // One wave per row; the row (after the residual add) stays in registers between the
-// sum-of-squares pass and the scaling pass.  NI = 16-byte items per lane.
+// sum-of-squares pass and the scaling pass.  NI = 16-byte items per lane.  Inputs are read once:
+// non-temporal loads.
 template <typename T, int NI>
 __global__ __launch_bounds__(256) void ksa_add_rmsnorm_kernel(const NormParams p) {
     using C = KsaCvt<T>;
@@ -41,9 +42,9 @@ __global__ __launch_bounds__(256) void ksa_add_rmsnorm_kernel(const NormParams p
         for (int j = 0; j < NI; ++j) {
             const int idx = lane + 64 * j;
             if (idx < items) {
-                r[j] = *reinterpret_cast<const u32x4*>(p.x + row * p.xs + 8 * idx);
+                r[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.x + row * p.xs + 8 * idx));
                 if (p.res) {
-                    const u32x4 q = *reinterpret_cast<const u32x4*>(p.res + row * p.rs + 8 * idx);
+                    const u32x4 q = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.res + row * p.rs + 8 * idx));
 #pragma unroll
                     for (int i = 0; i < 4; ++i)
                         r[j][i] = C::down2(C::lo(r[j][i]) + C::lo(q[i]), C::hi(r[j][i]) + C::hi(q[i]));
@@ -112,8 +113,8 @@ __global__ __launch_bounds__(256) void ksa_silu_mul_kernel(const ActParams p) {
     const int64_t row = blockIdx.x;
     const int idx = blockIdx.y * 256 + threadIdx.x;
     if (idx >= p.I / 8) return;
-    const u32x4 g = *reinterpret_cast<const u32x4*>(p.gate + row * p.gs + 8 * idx);
-    const u32x4 u = *reinterpret_cast<const u32x4*>(p.up + row * p.us + 8 * idx);
+    const u32x4 g = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.gate + row * p.gs + 8 * idx));
+    const u32x4 u = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.up + row * p.us + 8 * idx));
     u32x4 o;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
