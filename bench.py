@@ -186,6 +186,8 @@ def main():
                     help="also run the end-to-end decoder (random-init 4B shape: 36 layers, 3 Summary : 1 "
                          "full, batch 8, 32k-token prompt, 256 greedy steps) and report prefill and "
                          "decode tokens/s under 'e2e'")
+    ap.add_argument("--e2e-graph", action="store_true",
+                    help="replay the non-boundary decode steps of --e2e from a HIP graph")
     ap.add_argument("--e2e-batch", type=int, default=8)
     ap.add_argument("--e2e-prompt", type=int, default=32768)
     ap.add_argument("--e2e-new", type=int, default=256)
@@ -383,7 +385,7 @@ def main():
         for _ in range(args.e2e_new):
             nxt = logits[:, 0].argmax(-1, keepdim=True)
             n_boundary += cache.get_cur_chunk_size() == cfg.summary_chunk_size - 1
-            logits = model.decode_step(nxt, cache)
+            logits = model.decode_step_graph(nxt, cache) if args.e2e_graph else model.decode_step(nxt, cache)
         torch.cuda.synchronize()
         t_decode = time.perf_counter() - t0
         result["e2e"] = {
@@ -393,7 +395,7 @@ def main():
             "prefill_s": t_prefill, "prefill_tokens_per_s": args.e2e_batch * args.e2e_prompt / t_prefill,
             "decode_s": t_decode, "decode_ms_per_step": t_decode / args.e2e_new * 1e3,
             "decode_tokens_per_s": args.e2e_batch * args.e2e_new / t_decode,
-            "chunk_boundary_steps": int(n_boundary),
+            "chunk_boundary_steps": int(n_boundary), "decode_hip_graph": bool(args.e2e_graph),
             "hbm_allocated_gb": torch.cuda.max_memory_allocated() / 1e9,
         }
         del model, weights, cache, logits

@@ -23,9 +23,12 @@ from . import _lib
 
 
 def _move_rows(src: torch.Tensor, dst: torch.Tensor, nrows: int, src_start: int = 0,
-               dst_start: int = 0, src_index: Optional[torch.Tensor] = None) -> None:
+               dst_start: int = 0, src_index: Optional[torch.Tensor] = None,
+               dst_start_seq: Optional[torch.Tensor] = None) -> None:
     """dst[:, :, dst_start + i, :] <- src[:, :, src_index[i] | src_start + i, :] on the GPU.
-    src/dst are [bsz, heads, rows, D] with contiguous rows."""
+    src/dst are [bsz, heads, rows, D] with contiguous rows.  `dst_start_seq` (int32 [bsz] on the
+    GPU) replaces `dst_start` per sequence with values the kernel reads at run time, so a launch
+    recorded in a HIP graph can be replayed with other destination rows."""
     if nrows <= 0:
         return
     bsz, heads, _, D = dst.shape
@@ -38,7 +41,8 @@ def _move_rows(src: torch.Tensor, dst: torch.Tensor, nrows: int, src_start: int 
     with torch.cuda.device(dst.device):
         rc = _lib.lib().ksa_copy_rows(
             src.data_ptr(), dst.data_ptr(),
-            src_index.data_ptr() if src_index is not None else None, None,
+            src_index.data_ptr() if src_index is not None else None,
+            dst_start_seq.data_ptr() if dst_start_seq is not None else None,
             src_start, dst_start, nrows, bsz, heads, D,
             _lib.strides3(src, (0, 1, 2)), _lib.strides3(dst, (0, 1, 2)),
             _lib.stream_ptr(dst.device))

@@ -216,6 +216,8 @@ class KsaQwen3ForCausalLM:
         self.scaling = D ** -0.5
         emb = weights["embed_tokens"]
         self.dtype, self.device = emb.dtype, emb.device
+        self.inv_freq_dev = self.inv_freq.to(self.device)
+        self._graphs = {}
         self.lm_head = emb[: config.vocab_size] if config.tie_word_embeddings else weights["lm_head"]
 
     # ---- pieces ----------------------------------------------------------------------
@@ -227,7 +229,7 @@ class KsaQwen3ForCausalLM:
 
     def _rope_tables(self, position_ids):
         """cos, sin [1, L, D] in the model dtype from position ids [1, L] (computed in fp32)."""
-        freqs = position_ids[0].to(self.device).float()[:, None] * self.inv_freq.to(self.device)[None, :]
+        freqs = position_ids[0].to(self.device).float()[:, None] * self.inv_freq_dev[None, :]
         emb = torch.cat((freqs, freqs), dim=-1)
         return emb.cos().to(self.dtype)[None], emb.sin().to(self.dtype)[None]
 
@@ -333,6 +335,85 @@ class KsaQwen3ForCausalLM:
         cache.reset_chunk_counter()
         return self._logits(x[:, :1], delta[:, :1])
 
+    # ---- decode through a HIP graph ----------------------------------------------------
+    def _text_step_body(self, st, cache):
+        """One non-boundary decode step in a form that can be recorded once and replayed: every
+        per-step quantity (token ids, position, the cache row the new K/V go to, the attended row
+        range) is read from device tensors of `st`, never baked into a launch."""
+        cfg, ops = self.config, self.ops
+        cos, sin = self._rope_tables(st["pos"])
+        x = self.w["embed_tokens"][st["tok"]]
+        b = x.shape[0]
+        delta = None
+        for li, lw in enumerate(self.w["layers"]):
+            kind = 1 if cache.is_large_window[li] else 0
+            x, h = self._add_norm(delta, x, lw["input_layernorm"])
+            q, k, v = self._qkv(lw, h, None)
+            q, k, v = ops.pre_attention(q, k, v, lw["q_norm"], lw["k_norm"], cos, sin, cfg.rms_norm_eps)
+            cache._move_rows(k.transpose(1, 2), cache.key_cache[li], 1, dst_start_seq=st["cur"][kind, 0])
+            cache._move_rows(v.transpose(1, 2), cache.value_cache[li], 1, dst_start_seq=st["cur"][kind, 0])
+            attn = ops.decode(q.transpose(1, 2), cache.key_cache[li], cache.value_cache[li],
+                              st["cur"][kind, 1], st["cur"][kind, 2], self.scaling)
+            x, h = self._add_norm(F.linear(attn.reshape(b, 1, -1), lw["o_proj"]), x, lw["post_attention_layernorm"])
+            delta = self._mlp(lw, h)
+        return self._logits(x, delta)
+
+    @torch.no_grad()
+    def decode_step_graph(self, token_ids: torch.Tensor, cache):
+        """`decode_step` with the launches of a non-boundary step replayed from a HIP graph (about
+        400 launches per step otherwise cost more host time than GPU time).  Chunk-boundary steps
+        run as in `decode_step`.  The graph is recorded again when a cache buffer was reallocated.
+        The returned logits live in a buffer that the next call overwrites."""
+        cfg = self.config
+        C, S = cfg.summary_chunk_size, cfg.summary_token_num
+        if cache.get_cur_chunk_size() == C - 1:
+            return self.decode_step(token_ids, cache)
+        b = token_ids.shape[0]
+        Hkv, D = cfg.num_key_value_heads, cfg.head_dim
+        st = self._graphs.get(id(cache))
+        if st is None or st["batch"] != b:
+            st = {"batch": b, "graph": None, "ptrs": None,
+                  "tok": torch.zeros(b, 1, dtype=torch.long, device=self.device),
+                  "pos": torch.zeros(1, 1, dtype=torch.long, device=self.device),
+                  # [kind: small / large window][destination row, range start, range end][sequence]
+                  "cur": torch.zeros(2, 3, b, dtype=torch.int32, device=self.device)}
+            self._graphs = {id(cache): st}
+        p = cache.get_true_token_num() if cfg.summary_chunk_position_ids_type == "origin" \
+            else cache.get_cur_chunk_size()
+        # host bookkeeping of the step (may enlarge an append-only buffer), then this step's rows
+        rows = [None, None]
+        for li in range(cfg.num_hidden_layers):
+            kind = 1 if cache.is_large_window[li] else 0
+            if rows[kind] is None:
+                rows[kind] = cache._text_len[li] if kind else S + C - 1 - cache._chunk_buf_len[li]
+            cache.text_slots(li, b, Hkv, D, self.dtype, self.device)
+        vals = [[0, 0, 1], [0, 0, 1]]
+        for li in range(cfg.num_hidden_layers):
+            kind = 1 if cache.is_large_window[li] else 0
+            if rows[kind] is not None:
+                a, e = cache.attention_range(li)
+                vals[kind] = [rows[kind], a, e]
+                rows[kind] = None
+        # a fresh pageable host tensor: the runtime stages it before the call returns, so the host
+        # may run ahead of the GPU without overwriting values of a step still in flight
+        st["cur"].copy_(torch.tensor(vals, dtype=torch.int32).view(2, 3, 1))
+        st["tok"].copy_(token_ids.to(self.device))
+        st["pos"].fill_(p)
+        ptrs = tuple(t.data_ptr() for t in cache.key_cache + cache.value_cache)
+        if st["graph"] is None or st["ptrs"] != ptrs:
+            side = torch.cuda.Stream(device=self.device)
+            side.wait_stream(torch.cuda.current_stream(self.device))
+            with torch.cuda.stream(side):   # the step is idempotent: run it once before recording it
+                self._text_step_body(st, cache)
+            torch.cuda.current_stream(self.device).wait_stream(side)
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                st["logits"] = self._text_step_body(st, cache)
+            st["graph"], st["ptrs"] = g, ptrs
+        st["graph"].replay()
+        cache.reset_chunk_counter()
+        return st["logits"]
+
     # ---- driver ----------------------------------------------------------------------
     def forward(self, input_ids: torch.Tensor, cache=None):
         """Prefill when there is no (or an empty) cache, one decode step otherwise."""
@@ -342,10 +423,11 @@ class KsaQwen3ForCausalLM:
 
     @torch.no_grad()
     def generate(self, input_ids: torch.Tensor, max_new_tokens: int, forced: Optional[torch.Tensor] = None,
-                 return_logits: bool = False):
+                 return_logits: bool = False, use_graph: bool = False):
         """Greedy decoding.  Returns ids [b, n + max_new_tokens] (and the logits of every step,
         [b, max_new_tokens, vocab], on request).  `forced` [b, max_new_tokens] replaces the
-        arg-max token fed back at every step (teacher forcing, for comparing two runs)."""
+        arg-max token fed back at every step (teacher forcing, for comparing two runs).
+        `use_graph` replays the non-boundary decode steps from a HIP graph."""
         logits, cache = self.prefill(input_ids)
         out, steps = [], []
         for t in range(max_new_tokens):
@@ -355,6 +437,6 @@ class KsaQwen3ForCausalLM:
             out.append(nxt)
             if t + 1 < max_new_tokens:
                 feed = nxt if forced is None else forced[:, t:t + 1].to(self.device)
-                logits = self.decode_step(feed, cache)
+                logits = self.decode_step_graph(feed, cache) if use_graph else self.decode_step(feed, cache)
         ids = torch.cat([input_ids.to(self.device)] + out, dim=1)
         return (ids, torch.stack(steps, dim=1)) if return_logits else ids

@@ -167,3 +167,50 @@ def test_gpu_module_kernel_shape():
                       summary_sliding_chunk_num=[1, 1 << 20, 1], vocab_size=1000, summary_token_begin=1000)
     rel, agree = _gpu_vs_cpu(cfg, batch=2, n_prompt=300, n_new=120, seed=4, tol_rel=1.5e-2)
     print(f"max logit error {rel:.3e} of the logit scale, arg-max agreement {agree:.2f}")
+
+
+@pytest.mark.gpu
+def test_gpu_graph_decode_equals_eager_decode():
+    """The HIP-graph decode path against the eager one on the same inputs: 150 steps that cross a
+    chunk boundary and one reallocation of the append-only buffers (forcing a second recording),
+    every replay compared.  The two paths choose the decode kernel's split count differently
+    (the graph path cannot look at the row range on the host), so the logits agree to rounding,
+    not bit for bit: tolerance 1 % of the logit scale at every step."""
+    from ksa_amd.model import HipOps
+    cfg = tiny_config(summary_chunk_size=128, summary_token_num=8, head_dim=128, num_attention_heads=8,
+                      num_key_value_heads=2, hidden_size=256, intermediate_size=512, num_hidden_layers=4,
+                      summary_sliding_chunk_num=[1, 1 << 20, 1, 1 << 20], vocab_size=1000,
+                      summary_token_begin=1000)
+    w = init_weights(cfg, "cuda", torch.bfloat16, 7)
+    model = KsaQwen3ForCausalLM(cfg, w, HipOps())
+    ids = torch.randint(0, cfg.vocab_size, (2, 200), generator=torch.Generator().manual_seed(9))
+    n_new = 150
+    out_e, log_e = model.generate(ids, n_new, return_logits=True)
+    out_g, log_g = model.generate(ids, n_new, forced=out_e[:, 200:], return_logits=True, use_graph=True)
+    torch.cuda.synchronize()
+    err = (log_e - log_g).abs().amax(dim=(0, 2))
+    scale = log_e.abs().max().item()
+    print(f"graph vs eager: max logit difference {err.max().item() / scale:.3e} of the logit scale")
+    assert err.max().item() <= 1e-2 * scale, (err / scale).tolist()
+
+
+@pytest.mark.gpu
+def test_gpu_graph_decode_survives_buffer_growth():
+    """A small head-room makes the append-only text buffers grow during decoding, which moves
+    them; the graph path must notice and record again."""
+    from ksa_amd.model import HipOps
+    cfg = tiny_config(summary_chunk_size=128, summary_token_num=8, head_dim=128, num_attention_heads=8,
+                      num_key_value_heads=2, hidden_size=256, intermediate_size=512, num_hidden_layers=2,
+                      summary_sliding_chunk_num=[1, 1 << 20], vocab_size=1000, summary_token_begin=1000)
+    w = init_weights(cfg, "cuda", torch.bfloat16, 8)
+    ops = HipOps()
+
+    class SmallHeadroom(ops.cache_cls):
+        _APPEND_HEADROOM = 16
+    ops.cache_cls = SmallHeadroom
+    model = KsaQwen3ForCausalLM(cfg, w, ops)
+    ids = torch.randint(0, cfg.vocab_size, (1, 140), generator=torch.Generator().manual_seed(10))
+    out_e, log_e = model.generate(ids, 60, return_logits=True)
+    out_g, log_g = model.generate(ids, 60, forced=out_e[:, 140:], return_logits=True, use_graph=True)
+    err = (log_e - log_g).abs().amax(dim=(0, 2))
+    assert err.max().item() <= 1e-2 * log_e.abs().max().item(), err.tolist()
