@@ -326,12 +326,18 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
         // every text row of the tile has xa >= w_first * S and blo >= P >= thr
         const int thr = (prefix_mode && !mk.skip_old) ? min(w_first * mk.S, mk.P) : 0;
         const int nlim = thr / kTileN;  // tiles n < nlim end at or below thr
-        int lo = 0, hi = npart;         // first index with plist[i] >= nlim
-        while (lo < hi) {
-            const int mid = (lo + hi) >> 1;
-            if (plist[mid] < nlim) lo = mid + 1; else hi = mid;
+        // number of entries of the ascending list below nlim (at most nlim of them): counted by
+        // the whole wave, 128 entries per round of independent loads, instead of a binary search
+        // whose dependent loads would cost several microseconds at the start of every workgroup
+        const int lim = min(npart, nlim);
+        int cnt = 0;
+        for (int base = 0; base < lim; base += 128) {
+            const int i0 = base + lane, i1 = base + 64 + lane;
+            const int e0 = i0 < lim ? plist[i0] : nlim;
+            const int e1 = i1 < lim ? plist[i1] : nlim;
+            cnt += __popcll(__ballot(e0 < nlim)) + __popcll(__ballot(e1 < nlim));
         }
-        nquick = lo;
+        nquick = cnt;
     }
     const bool last_full_cut = nfull > 0 && (flist[nfull - 1] + 1) * kTileN > mk.Sk;
     const int nfull_a = nfull - (last_full_cut ? 1 : 0);
