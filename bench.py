@@ -169,6 +169,9 @@ def main():
     ap.add_argument("--sliding-chunk-num", type=int, default=4)
     ap.add_argument("--decode-batch", type=int, default=64)
     ap.add_argument("--decode-splits", type=int, default=0, help="0 = library heuristic")
+    ap.add_argument("--idle", type=float, default=1.0, metavar="SECONDS",
+                    help="idle time before each timed section, so that every section starts from the "
+                         "same (idle) power state instead of the one its predecessor left")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--skip-decode", action="store_true")
     ap.add_argument("--skip-prefill", action="store_true")
@@ -216,6 +219,7 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic (seed 0; q,k,v ~ N(0,1)/sqrt(128) for prefill, N(0,1) for decode)",
         "device": torch.cuda.get_device_name(0), "cu_count": _lib.lib().ksa_device_cu_count(),
+        "idle_before_each_section_s": args.idle,
     }
 
     if args.calibrate_copy:
@@ -289,6 +293,8 @@ def main():
 
     # ------------------------------------------------------------------ decode
     if not args.skip_decode:
+        torch.cuda.synchronize()
+        time.sleep(args.idle)
         Bz = args.decode_batch
         n_chunks_done = 1024
         ws = W * C
@@ -333,6 +339,8 @@ def main():
 
     # ------------------------------------------------------------------ pre-attention step
     if not args.skip_pre_attention:
+        torch.cuda.synchronize()
+        time.sleep(args.idle)
         chunks = args.prefill_chunks
         Sp = chunks * (C + S)
         g = torch.Generator(device=dev).manual_seed(2)
