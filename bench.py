@@ -250,6 +250,8 @@ def main():
         def step():
             ksa_amd.summary_attn_func(q, k, v, C, S, W, summary_pos=sp)
 
+        torch.cuda.synchronize()
+        time.sleep(args.idle)
         wall, dev_ms = time_region(step, args.steps, args.warmup)
         ms = wall * 1e3 / args.steps
         kern_ms = dev_ms / args.steps
