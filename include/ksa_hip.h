@@ -141,6 +141,19 @@ int ksa_silu_mul(const void* gate, const void* up, void* out, long long rows, in
                  long long gate_row_stride, long long up_row_stride, long long out_row_stride,
                  int dtype, void* stream);
 
+/* y = x W^T for at most 16 rows of x (decode steps), bound by the weight bytes.
+ * Replaces torch.nn.functional.linear at the projections of a decode step (HF:628-641 q/k/v and
+ * o projections, HF:507-514 MLP, HF:1338 lm_head), bias-free as in the reference's config.
+ *   x [M, K], w [N, K], out [M, N], 16-bit, row strides in elements (x, w: multiples of 8);
+ *   K a multiple of 32; fp32 accumulation, one rounding at the end.
+ * ksplit > 1 splits K over workgroups (ksa_gemm_rows_auto_splits) and needs
+ * ksa_gemm_rows_workspace_bytes(N, ksplit) bytes of device workspace. */
+int ksa_gemm_rows_auto_splits(int N, int K);
+size_t ksa_gemm_rows_workspace_bytes(int N, int ksplit);
+int ksa_gemm_rows(const void* x, const void* w, void* out, int M, int N, int K, long long x_row_stride,
+                  long long w_row_stride, long long out_row_stride, int dtype, int ksplit,
+                  void* workspace, size_t workspace_bytes, void* stream);
+
 /* Measurement aid (no counterpart in the reference): launches a pure stream of bf16 MFMA
  * 32x32x16 instructions (blocks x waves_per_block waves, 16 * iters instructions each, operands
  * random or all zero) and returns the floating-point operations of the launch in *flop.  Timed

@@ -15,10 +15,11 @@ from .decode import decode_attention_forward, ksa_decode  # noqa: E402
 from .cache import Qwen3RingBufferCache  # noqa: E402
 from .pre import pre_attention  # noqa: E402
 from .elementwise import add_rmsnorm, silu_mul  # noqa: E402
+from .gemm import linear_rows  # noqa: E402
 from .model import KsaQwen3Config, KsaQwen3ForCausalLM, init_weights  # noqa: E402
 
 __all__ = [
     "KsaError", "SUMMARY_ATTN_CACHE", "compute_block_sparsity", "summary_attn_func",
-    "decode_attention_forward", "ksa_decode", "Qwen3RingBufferCache", "pre_attention", "add_rmsnorm", "silu_mul",
+    "decode_attention_forward", "ksa_decode", "Qwen3RingBufferCache", "pre_attention", "add_rmsnorm", "silu_mul", "linear_rows",
     "KsaQwen3Config", "KsaQwen3ForCausalLM", "init_weights",
 ]

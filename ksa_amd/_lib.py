@@ -33,6 +33,9 @@ _SIGNATURES = {
     "ksa_add_rmsnorm": (_int, [_vp] * 5 + [ctypes.c_longlong, _int] + [ctypes.c_longlong] * 4
                         + [_int, ctypes.c_float, _vp]),
     "ksa_silu_mul": (_int, [_vp] * 3 + [ctypes.c_longlong, _int] + [ctypes.c_longlong] * 3 + [_int, _vp]),
+    "ksa_gemm_rows_auto_splits": (_int, [_int, _int]),
+    "ksa_gemm_rows_workspace_bytes": (ctypes.c_size_t, [_int, _int]),
+    "ksa_gemm_rows": (_int, [_vp] * 3 + [_int] * 3 + [ctypes.c_longlong] * 3 + [_int, _int, _vp, ctypes.c_size_t, _vp]),
     "ksa_probe_mfma_stream": (_int, [_vp] + [_int] * 4 + [ctypes.POINTER(ctypes.c_double), _vp]),
     "ksa_debug_count_visible": (ctypes.c_longlong, [ctypes.c_longlong] * 3 + [_int] * 7),
 }

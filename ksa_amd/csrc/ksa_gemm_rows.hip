@@ -1,0 +1,161 @@
+// y = x W^T for a handful of rows (decode steps: one row per sequence), gfx950.
+//
+// The projections of a decode step (examples/pretrain/hf_template/modeling_qwen3sa.py: q/k/v
+// and o projections :628-641, :879; the MLP :507-514; lm_head :1338, :1395) multiply at most a
+// few rows by a weight matrix that has to be streamed from HBM once: the step is bound by the
+// weight bytes.  A wave owns 16 output columns (16 rows of W, each K elements long) and a
+// slice of K; a weight fragment goes from global memory straight into the A operand of a
+// 16x16x32 MFMA (lane = (row of W, quarter of the 32-wide K step): 16 contiguous bytes per lane,
+// 64 contiguous bytes per row and instruction), the rows of x are the B operand.  The K slices
+// of a workgroup's four waves are added through LDS; with more than one K split per column tile
+// the fp32 partial sums go to a workspace and a second kernel adds and rounds them.
+#include <hip/hip_runtime.h>
+
+#include "ksa_api_internal.h"
+#include "ksa_cvt.h"
+
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+struct GemmParams {
+    const uint16_t* x;   // [M, K], row stride xs
+    const uint16_t* w;   // [N, K], row stride ws
+    uint16_t* out;       // [M, N], row stride os
+    float* part;         // [ksplit, 16, N] when ksplit > 1
+    int64_t xs, ws, os;
+    int M, N, K, ksplit;
+};
+
+template <typename T>
+__device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c);
+template <>
+__device__ __forceinline__ f32x4 mfma16<KsaBf16>(u32x4 a, u32x4 b, f32x4 c) {
+    typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
+                                                   0, 0, 0);
+}
+template <>
+__device__ __forceinline__ f32x4 mfma16<KsaF16>(u32x4 a, u32x4 b, f32x4 c) {
+    typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c,
+                                                  0, 0, 0);
+}
+
+constexpr int kUnroll = 8;  // weight fragments in flight per lane (8 x 16 bytes)
+
+// grid: (column tiles of 16, K splits); block: 4 waves, each a quarter of the split's K steps
+template <typename T>
+__global__ __launch_bounds__(256) void ksa_gemm_rows_kernel(const GemmParams p) {
+    using C = KsaCvt<T>;
+    __shared__ float red[4][16][17];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int r = lane & 15;   // row of W inside the tile (A operand) / row of x (B operand)
+    const int kq = lane >> 4;  // which 8 of the 32 K elements of a step
+    const int n0 = blockIdx.x * 16;
+    const int steps = p.K / 32;
+    // K steps of this wave: split blockIdx.y of ksplit, then wave quarter
+    const int per_split = (steps + p.ksplit - 1) / p.ksplit;
+    const int s_begin = blockIdx.y * per_split;
+    const int s_end = min(steps, s_begin + per_split);
+    const int per_wave = (max(s_end - s_begin, 0) + 3) / 4;
+    const int w_begin = s_begin + wave * per_wave;
+    const int w_end = min(s_end, w_begin + per_wave);
+
+    const int nrow = min(n0 + r, p.N - 1);
+    const uint16_t* wp = p.w + (int64_t)nrow * p.ws + 8 * kq;
+    // rows of x beyond M repeat the last one: their columns of the product are never stored
+    const uint16_t* xp = p.x + (int64_t)min(r, p.M - 1) * p.xs + 8 * kq;
+
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    // batches of kUnroll steps, all loads of a batch issued before its first MFMA; steps past
+    // the end of the slice repeat the last step with a zero weight fragment
+    for (int s = w_begin; s < w_end; s += kUnroll) {
+        u32x4 a[kUnroll], b[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const int su = min(s + u, w_end - 1);
+            a[u] = *reinterpret_cast<const u32x4*>(wp + 32 * su);
+            b[u] = *reinterpret_cast<const u32x4*>(xp + 32 * su);
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            if (s + u >= w_end) a[u] = u32x4{0u, 0u, 0u, 0u};
+            acc = mfma16<T>(a[u], b[u], acc);
+        }
+    }
+    // C layout of the 16x16 tile: lane holds column (row of x) lane % 16, rows (of W) 4 * (lane / 16) + i
+#pragma unroll
+    for (int i = 0; i < 4; ++i) red[wave][4 * kq + i][r] = acc[i];
+    __syncthreads();
+    // thread t < 256: output element (x row m = t % 16, W row j = t / 16)
+    const int m = threadIdx.x & 15, j = threadIdx.x >> 4;
+    const float v = red[0][j][m] + red[1][j][m] + red[2][j][m] + red[3][j][m];
+    const int n = n0 + j;
+    if (m < p.M && n < p.N) {
+        if (p.ksplit == 1) p.out[(int64_t)m * p.os + n] = C::down(v);
+        else p.part[((int64_t)blockIdx.y * 16 + m) * p.N + n] = v;
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void ksa_gemm_rows_reduce_kernel(const GemmParams p) {
+    using C = KsaCvt<T>;
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e >= (int64_t)p.M * p.N) return;
+    const int m = (int)(e / p.N), n = (int)(e % p.N);
+    float v = 0.f;
+    for (int sp = 0; sp < p.ksplit; ++sp) v += p.part[((int64_t)sp * 16 + m) * p.N + n];
+    p.out[(int64_t)m * p.os + n] = C::down(v);
+}
+
+template <typename T>
+int launch_gemm(const GemmParams& p, hipStream_t st) {
+    dim3 grid((p.N + 15) / 16, p.ksplit);
+    hipLaunchKernelGGL(ksa_gemm_rows_kernel<T>, grid, dim3(256), 0, st, p);
+    if (p.ksplit > 1) {
+        const int64_t n = (int64_t)p.M * p.N;
+        hipLaunchKernelGGL(ksa_gemm_rows_reduce_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, p);
+    }
+    return ksa_check_launch();
+}
+
+}  // namespace
+
+// K splits that give about four workgroups per CU (256 CUs) without slices shorter than 16 steps
+extern "C" int ksa_gemm_rows_auto_splits(int N, int K) {
+    if (N <= 0 || K <= 0) return 1;
+    const int tiles = (N + 15) / 16;
+    int sp = (1024 + tiles - 1) / tiles;
+    const int cap = K / 32 / 16 > 1 ? K / 32 / 16 : 1;
+    if (sp > cap) sp = cap;
+    if (sp > 16) sp = 16;
+    return sp < 1 ? 1 : sp;
+}
+
+extern "C" size_t ksa_gemm_rows_workspace_bytes(int N, int ksplit) {
+    return ksplit > 1 ? (size_t)ksplit * 16 * (size_t)N * sizeof(float) : 0;
+}
+
+extern "C" int ksa_gemm_rows(const void* x, const void* w, void* out, int M, int N, int K, long long x_row_stride,
+                             long long w_row_stride, long long out_row_stride, int dtype, int ksplit,
+                             void* workspace, size_t workspace_bytes, void* stream) {
+    if (!x || !w || !out) return KSA_ERR_NULL;
+    if (M <= 0 || M > 16 || N <= 0 || K <= 0 || K % 32 != 0 || ksplit < 1 || ksplit > 64) return KSA_ERR_INVALID;
+    if (dtype != KSA_DTYPE_BF16 && dtype != KSA_DTYPE_F16) return KSA_ERR_UNSUPPORTED;
+    if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w)) & 15) return KSA_ERR_ALIGN;
+    if (x_row_stride % 8 || w_row_stride % 8) return KSA_ERR_ALIGN;
+    GemmParams p{};
+    p.x = (const uint16_t*)x;
+    p.w = (const uint16_t*)w;
+    p.out = (uint16_t*)out;
+    p.xs = x_row_stride, p.ws = w_row_stride, p.os = out_row_stride;
+    p.M = M, p.N = N, p.K = K, p.ksplit = ksplit;
+    if (ksplit > 1) {
+        if (!workspace || workspace_bytes < ksa_gemm_rows_workspace_bytes(N, ksplit)) return KSA_ERR_WORKSPACE;
+        p.part = (float*)workspace;
+    }
+    return dtype == KSA_DTYPE_BF16 ? launch_gemm<KsaBf16>(p, (hipStream_t)stream)
+                                   : launch_gemm<KsaF16>(p, (hipStream_t)stream);
+}

@@ -14,7 +14,7 @@ Differences from the reference, on purpose:
 * any batch size (the reference refuses batch > 1 at :753; its cache tensors and counters are
   already batch-shaped, all sequences of a batch have the same length);
 * weights are plain tensors (fused q|k|v and gate|up matrices), not nn.Modules; the GEMMs are
-  torch matmuls (hipBLASLt), everything else (pre-attention, attention, cache rows, residual add +
+  torch matmuls (hipBLASLt) except for the few rows of a decode step (`ksa_gemm_rows`), everything else (pre-attention, attention, cache rows, residual add +
   RMSNorm, SiLU-mul) is this package's kernels;
 * a "full attention" layer is, as in the reference's inference model, a Summary layer whose
   window is larger than any sequence (append-only text cache, :114-115, :232-242);
@@ -128,16 +128,26 @@ class HipOps:
     """The attention-side operators of the model, bound to this package's HIP kernels."""
 
     def __init__(self):
-        from . import cache, decode, elementwise, pre, prefill
+        from . import cache, decode, elementwise, gemm, pre, prefill
         self.cache_cls = cache.Qwen3RingBufferCache
         self.pre_attention = pre.pre_attention
         self.summary_attn_func = prefill.summary_attn_func
         self.add_rmsnorm = elementwise.add_rmsnorm
         self.silu_mul = elementwise.silu_mul
         self._decode = decode.ksa_decode
+        self._linear_rows = gemm.linear_rows
+        self._max_rows = gemm.MAX_ROWS
 
     def decode(self, q, kbuf, vbuf, start, end, scale):
         return self._decode(q, kbuf, vbuf, start, end, scale=scale)
+
+    def linear(self, x, weight):
+        """x W^T: the weight-streaming kernel for the few rows of a decode step, the library
+        GEMM otherwise."""
+        rows = x.numel() // x.shape[-1]
+        if rows <= self._max_rows and x.shape[-1] % 32 == 0:
+            return self._linear_rows(x, weight)
+        return F.linear(x, weight)
 
 
 def expand_with_summary_tokens(input_ids: torch.Tensor, config: KsaQwen3Config):
@@ -237,10 +247,10 @@ class KsaQwen3ForCausalLM:
         """Projection outputs as strided views q [b, L, Hq, D], k, v [b, L, Hkv, D]."""
         cfg = self.config
         D, Hq, Hkv = cfg.head_dim, cfg.num_attention_heads, cfg.num_key_value_heads
-        qkv = F.linear(h, lw["qkv_proj"])
+        qkv = self.ops.linear(h, lw["qkv_proj"])
         if (cfg.summary_independent_parameters and cfg.mix_coeff != 0 and summary_rows is not None
                 and summary_rows.numel() > 0):
-            qkv[:, summary_rows] = F.linear(h[:, summary_rows], lw["qkv_proj_summary"])
+            qkv[:, summary_rows] = self.ops.linear(h[:, summary_rows], lw["qkv_proj_summary"])
         b, L, _ = qkv.shape
         q = qkv[..., : Hq * D].view(b, L, Hq, D)
         k = qkv[..., Hq * D: (Hq + Hkv) * D].view(b, L, Hkv, D)
@@ -248,13 +258,13 @@ class KsaQwen3ForCausalLM:
         return q, k, v
 
     def _mlp(self, lw, x):
-        gu = F.linear(x, lw["gate_up_proj"])
+        gu = self.ops.linear(x, lw["gate_up_proj"])
         I = self.config.intermediate_size
-        return F.linear(self.ops.silu_mul(gu[..., :I], gu[..., I:]), lw["down_proj"])
+        return self.ops.linear(self.ops.silu_mul(gu[..., :I], gu[..., I:]), lw["down_proj"])
 
     def _logits(self, x_last, delta_last):
         _, h = self._add_norm(delta_last, x_last, self.w["norm"])
-        return F.linear(h, self.lm_head)[..., : self.config.vocab_size]
+        return self.ops.linear(h, self.lm_head)[..., : self.config.vocab_size]
 
     # ---- prefill ---------------------------------------------------------------------
     @torch.no_grad()
@@ -278,7 +288,7 @@ class KsaQwen3ForCausalLM:
             q, k, v = ops.pre_attention(q, k, v, lw["q_norm"], lw["k_norm"], cos, sin, cfg.rms_norm_eps,
                                         k_out=k_slot, v_out=v_slot)
             attn, _ = ops.summary_attn_func(q, k, v, C, S, self.scns[li], summary_pos=is_sum)
-            x, h = self._add_norm(F.linear(attn.reshape(b, L, -1), lw["o_proj"]), x, lw["post_attention_layernorm"])
+            x, h = self._add_norm(ops.linear(attn.reshape(b, L, -1), lw["o_proj"]), x, lw["post_attention_layernorm"])
             delta = self._mlp(lw, h)
         cache.reorganize_after_prefill(is_sum[None])
         last_text = L - 1 if (L % (C + S)) != 0 else L - 1 - S   # the last prompt token's slot
@@ -329,7 +339,7 @@ class KsaQwen3ForCausalLM:
                 sum_out = ops.decode(qh[:, :, 1:], k_cs, v_cs, 0, k_cs.shape[2], self.scaling)
                 cache.update_summary(kh[:, :, 1:], vh[:, :, 1:], li)
                 attn = torch.cat([text_out, sum_out], dim=1)
-            x, h = self._add_norm(F.linear(attn.reshape(b, ids.shape[1], -1), lw["o_proj"]), x,
+            x, h = self._add_norm(ops.linear(attn.reshape(b, ids.shape[1], -1), lw["o_proj"]), x,
                                   lw["post_attention_layernorm"])
             delta = self._mlp(lw, h)
         cache.reset_chunk_counter()
@@ -354,7 +364,7 @@ class KsaQwen3ForCausalLM:
             cache._move_rows(v.transpose(1, 2), cache.value_cache[li], 1, dst_start_seq=st["cur"][kind, 0])
             attn = ops.decode(q.transpose(1, 2), cache.key_cache[li], cache.value_cache[li],
                               st["cur"][kind, 1], st["cur"][kind, 2], self.scaling)
-            x, h = self._add_norm(F.linear(attn.reshape(b, 1, -1), lw["o_proj"]), x, lw["post_attention_layernorm"])
+            x, h = self._add_norm(ops.linear(attn.reshape(b, 1, -1), lw["o_proj"]), x, lw["post_attention_layernorm"])
             delta = self._mlp(lw, h)
         return self._logits(x, delta)
 

@@ -44,6 +44,7 @@ class OracleOps:
             res.append(val)
         return tuple(res)
 
+    linear = staticmethod(torch.nn.functional.linear)
     add_rmsnorm = staticmethod(cpu_path.add_rmsnorm)
     silu_mul = staticmethod(cpu_path.silu_mul)
 
