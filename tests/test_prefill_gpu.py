@@ -368,3 +368,46 @@ def test_prefill_reference_far_too_high(wave_rows):
     err = np.abs(got[rows] - want).max()
     assert err <= ATOL * max(1.0, np.abs(want).max()), err
     assert np.abs(lse[:, rows] - wlse).max() <= 0.1 + 1e-3 * np.abs(wlse).max()
+
+
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_prefill_random_shapes(seed, monkeypatch):
+    """Twelve random small problems per seed - chunk sizes that are no power of two, summary
+    counts 1..8, windows 0..unbounded, head_dim 64 / 128, group sizes 1..6, all three ways of
+    passing the summaries, both dtypes, every workgroup shape - each against the oracle."""
+    import ksa_amd
+    rng = np.random.default_rng(seed)
+    dev = torch.device("cuda")
+    for ci in range(12):
+        C = int(rng.choice([4, 8, 16, 32, 64, 128, 128, 100, 24]))
+        S = min(int(rng.choice([1, 2, 4, 8, 8, 3, 5])), C)
+        W = int(rng.choice([0, 1, 2, 3, 4, 7, 1000]))
+        D = int(rng.choice([64, 128, 128]))
+        Hkv = int(rng.choice([1, 2, 3]))
+        Hq = Hkv * int(rng.choice([1, 2, 3, 4, 6]))
+        Sq = int(rng.integers(1, 2200))
+        mode = str(rng.choice(["prefix", "prefix", "inline", "physical"]))
+        skip = bool(rng.integers(0, 2))
+        dtype = torch.bfloat16 if rng.integers(0, 4) else torch.float16
+        shape = str(rng.choice(["", "32", "64"]))
+        if shape:
+            monkeypatch.setenv("KSA_PREFILL_ROWS_PER_WAVE", shape)
+        else:
+            monkeypatch.delenv("KSA_PREFILL_ROWS_PER_WAVE", raising=False)
+        q, k, v = make_qkv(Sq, Hq, Hkv, D, seed=seed * 100 + ci, scaled=bool(rng.integers(0, 2)))
+        q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
+        sp = O.summary_positions(Sq, C, S)
+        case = (seed, ci, Sq, Hq, Hkv, D, C, S, W, mode, skip, str(dtype), shape)
+        kk, vv, spt, osp = k, v, torch.as_tensor(sp, device=dev), sp
+        if mode == "inline":
+            spt, osp = None, None
+        elif mode == "physical":
+            st = torch.as_tensor(sp)
+            kk, vv, spt = torch.cat([k[st], k]), torch.cat([v[st], v]), None
+        out, lse = ksa_amd.summary_attn_func(q[None].to(dev), kk[None].to(dev), vv[None].to(dev), C, S, W,
+                                             summary_pos=spt, skip_old_summary=skip, return_lse=True)
+        want, wlse = c_oracle.attention_rows(to_np(q), to_np(k), to_np(v), C, S, W, summary_pos=osp, skip_old=skip)
+        got = to_np(out[0])
+        assert np.isfinite(got).all(), case
+        assert np.abs(got - want).max() <= ATOL * max(1.0, np.abs(want).max()), case
+        assert np.abs(to_np(lse[0]) - wlse).max() <= 5e-2, case
