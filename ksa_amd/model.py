@@ -14,8 +14,9 @@ Differences from the reference, on purpose:
 * any batch size (the reference refuses batch > 1 at :753; its cache tensors and counters are
   already batch-shaped, all sequences of a batch have the same length);
 * weights are plain tensors (fused q|k|v and gate|up matrices), not nn.Modules; the GEMMs are
-  torch matmuls (hipBLASLt) except for the few rows of a decode step (`ksa_gemm_rows`), everything else (pre-attention, attention, cache rows, residual add +
-  RMSNorm, SiLU-mul) is this package's kernels;
+  torch matmuls (hipBLASLt) except for the few rows of a decode step (`ksa_gemm_rows`);
+  everything else (pre-attention, attention, cache rows, residual add + RMSNorm, SiLU-mul) is
+  this package's kernels;
 * a "full attention" layer is, as in the reference's inference model, a Summary layer whose
   window is larger than any sequence (append-only text cache, :114-115, :232-242);
 * `summary_independent_parameters` is supported for mix_coeff 0 and 1 (the reference's default
