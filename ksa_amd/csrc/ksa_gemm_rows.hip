@@ -3,12 +3,12 @@
 // The projections of a decode step (examples/pretrain/hf_template/modeling_qwen3sa.py: q/k/v
 // and o projections :628-641, :879; the MLP :507-514; lm_head :1338, :1395) multiply at most a
 // few rows by a weight matrix that has to be streamed from HBM once: the step is bound by the
-// weight bytes.  A wave owns 16 output columns (16 rows of W, each K elements long) and a
-// slice of K; a weight fragment goes from global memory straight into the A operand of a
-// 16x16x32 MFMA (lane = (row of W, quarter of the 32-wide K step): 16 contiguous bytes per lane,
-// 64 contiguous bytes per row and instruction), the rows of x are the B operand.  The K slices
-// of a workgroup's four waves are added through LDS; with more than one K split per column tile
-// the fp32 partial sums go to a workspace and a second kernel adds and rounds them.
+// weight bytes.  A wave owns 16 output columns (16 rows of W, each K elements long); a weight
+// fragment goes from global memory straight into the A operand of a 16x16x32 MFMA (lane = (row
+// of W, quarter of the 32-wide K step): 16 contiguous bytes per lane, 64 contiguous bytes per
+// row and instruction), the rows of x, staged in LDS, are the B operand.  With more than one K
+// split per column tile the fp32 partial sums go to a workspace and a second kernel adds and
+// rounds them.
 #include <hip/hip_runtime.h>
 
 #include "ksa_api_internal.h"
@@ -42,60 +42,70 @@ __device__ __forceinline__ f32x4 mfma16<KsaF16>(u32x4 a, u32x4 b, f32x4 c) {
                                                   0, 0, 0);
 }
 
-constexpr int kUnroll = 8;  // weight fragments in flight per lane (8 x 16 bytes)
+constexpr int kChunkSteps = 16;                 // K steps (of 32) per staged chunk of x
+constexpr int kChunkK = 32 * kChunkSteps;       // 512 elements of K
+constexpr int kRowB = (kChunkK + 8) * 2;        // padded LDS row of x in bytes (conflict-free b128 reads)
 
-// grid: (column tiles of 16, K splits); block: 4 waves, each a quarter of the split's K steps
+// grid: (tiles of 64 output columns, K splits); block: 4 waves, each 16 columns over the whole K
+// slice.  Per chunk of 512 K elements a wave first requests its 16 weight fragments (16 x 16
+// bytes per lane in flight), the workgroup copies the chunk of x into LDS once, and the MFMAs
+// then take their B operands from there: x is fetched once per 64 columns instead of once per
+// wave and step, which is what held a first version of this kernel at 60 % of the rate below.
 template <typename T>
 __global__ __launch_bounds__(256) void ksa_gemm_rows_kernel(const GemmParams p) {
     using C = KsaCvt<T>;
-    __shared__ float red[4][16][17];
+    __shared__ __attribute__((aligned(16))) unsigned char xs[2][16 * kRowB];
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int r = lane & 15;   // row of W inside the tile (A operand) / row of x (B operand)
     const int kq = lane >> 4;  // which 8 of the 32 K elements of a step
-    const int n0 = blockIdx.x * 16;
+    const int n0 = (blockIdx.x * 4 + wave) * 16;
     const int steps = p.K / 32;
-    // K steps of this wave: split blockIdx.y of ksplit, then wave quarter
     const int per_split = (steps + p.ksplit - 1) / p.ksplit;
     const int s_begin = blockIdx.y * per_split;
     const int s_end = min(steps, s_begin + per_split);
-    const int per_wave = (max(s_end - s_begin, 0) + 3) / 4;
-    const int w_begin = s_begin + wave * per_wave;
-    const int w_end = min(s_end, w_begin + per_wave);
 
     const int nrow = min(n0 + r, p.N - 1);
     const uint16_t* wp = p.w + (int64_t)nrow * p.ws + 8 * kq;
     // rows of x beyond M repeat the last one: their columns of the product are never stored
-    const uint16_t* xp = p.x + (int64_t)min(r, p.M - 1) * p.xs + 8 * kq;
+    const int xrow = min(r, p.M - 1);
 
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-    // batches of kUnroll steps, all loads of a batch issued before its first MFMA; steps past
-    // the end of the slice repeat the last step with a zero weight fragment
-    for (int s = w_begin; s < w_end; s += kUnroll) {
-        u32x4 a[kUnroll], b[kUnroll];
+    int buf = 0;
+    for (int c0 = s_begin; c0 < s_end; c0 += kChunkSteps) {
+        const int nst = min(kChunkSteps, s_end - c0);
+        u32x4 a[kChunkSteps];
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            const int su = min(s + u, w_end - 1);
-            a[u] = *reinterpret_cast<const u32x4*>(wp + 32 * su);
-            b[u] = *reinterpret_cast<const u32x4*>(xp + 32 * su);
+        for (int u = 0; u < kChunkSteps; ++u) a[u] = *reinterpret_cast<const u32x4*>(wp + 32 * min(c0 + u, s_end - 1));
+        // x[0:M][32 c0 .. 32 (c0 + nst)) -> LDS, 16 bytes per thread and pass
+        for (int e = threadIdx.x; e < p.M * (kChunkK / 8); e += 256) {
+            const int m = e / (kChunkK / 8), j = e % (kChunkK / 8);
+            if (j < nst * 4)
+                *reinterpret_cast<u32x4*>(xs[buf] + m * kRowB + 16 * j) =
+                    *reinterpret_cast<const u32x4*>(p.x + (int64_t)m * p.xs + 32 * c0 + 8 * j);
         }
+        // (one barrier per chunk is enough with two buffers: nobody passes the next chunk's
+        // barrier before everybody has finished reading this one)
+        __syncthreads();
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            if (s + u >= w_end) a[u] = u32x4{0u, 0u, 0u, 0u};
-            acc = mfma16<T>(a[u], b[u], acc);
+        for (int u = 0; u < kChunkSteps; ++u) {
+            if (u < nst) {
+                const u32x4 b = *reinterpret_cast<const u32x4*>(xs[buf] + xrow * kRowB + 64 * u + 16 * kq);
+                acc = mfma16<T>(a[u], b, acc);
+            }
         }
+        buf ^= 1;
     }
     // C layout of the 16x16 tile: lane holds column (row of x) lane % 16, rows (of W) 4 * (lane / 16) + i
+    if (r < p.M) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) red[wave][4 * kq + i][r] = acc[i];
-    __syncthreads();
-    // thread t < 256: output element (x row m = t % 16, W row j = t / 16)
-    const int m = threadIdx.x & 15, j = threadIdx.x >> 4;
-    const float v = red[0][j][m] + red[1][j][m] + red[2][j][m] + red[3][j][m];
-    const int n = n0 + j;
-    if (m < p.M && n < p.N) {
-        if (p.ksplit == 1) p.out[(int64_t)m * p.os + n] = C::down(v);
-        else p.part[((int64_t)blockIdx.y * 16 + m) * p.N + n] = v;
+        for (int i = 0; i < 4; ++i) {
+            const int n = n0 + 4 * kq + i;
+            if (n < p.N) {
+                if (p.ksplit == 1) p.out[(int64_t)r * p.os + n] = C::down(acc[i]);
+                else p.part[((int64_t)blockIdx.y * 16 + r) * p.N + n] = acc[i];
+            }
+        }
     }
 }
 
@@ -112,7 +122,7 @@ __global__ __launch_bounds__(256) void ksa_gemm_rows_reduce_kernel(const GemmPar
 
 template <typename T>
 int launch_gemm(const GemmParams& p, hipStream_t st) {
-    dim3 grid((p.N + 15) / 16, p.ksplit);
+    dim3 grid((p.N + 63) / 64, p.ksplit);
     hipLaunchKernelGGL(ksa_gemm_rows_kernel<T>, grid, dim3(256), 0, st, p);
     if (p.ksplit > 1) {
         const int64_t n = (int64_t)p.M * p.N;
@@ -123,11 +133,11 @@ int launch_gemm(const GemmParams& p, hipStream_t st) {
 
 }  // namespace
 
-// K splits that give about four workgroups per CU (256 CUs) without slices shorter than 16 steps
+// K splits that give about two workgroups per CU (256 CUs) without slices shorter than one chunk
 extern "C" int ksa_gemm_rows_auto_splits(int N, int K) {
     if (N <= 0 || K <= 0) return 1;
-    const int tiles = (N + 15) / 16;
-    int sp = (1024 + tiles - 1) / tiles;
+    const int tiles = (N + 63) / 64;
+    int sp = (512 + tiles - 1) / tiles;
     const int cap = K / 32 / 16 > 1 ? K / 32 / 16 : 1;
     if (sp > cap) sp = cap;
     if (sp > 16) sp = 16;
