@@ -294,3 +294,29 @@ def test_ring_buffer_known_answers():
     r2.reorganize_after_prefill(np.arange(2 * 136 + 5), O.summary_positions(2 * 136 + 5, C, S))
     assert (r2.nv, r2.ptr, r2.cbl) == (256, 256, 5)
     assert r2.attention_range() == (136 - 5, 136 + 256)
+
+
+def test_known_answers_fixture():
+    """tests/golden/known_answers.json against the oracle: allowed-pair totals of all three
+    configurations by the closed-form row counts (no tiles involved), tile totals of cfg 0 by the
+    C index builder."""
+    import json
+    import os
+    ka = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "known_answers.json")))
+    C, S = ka["C"], ka["S"]
+    B = C + S
+    for name, cfg in ka["configs"].items():
+        Sq = cfg["Sq"]
+        rows = np.arange(Sq)
+        c, o = rows // B, rows % B
+        for W in (3, 4):
+            text = S * np.maximum(0, c - W) + C * np.minimum(c, W) + o + 1
+            summ = C + (o - C) + 1
+            pairs = int(np.where(o < C, text, summ).sum())
+            assert pairs == cfg[f"W{W}"]["pairs"], (name, W)
+            assert cfg["P"] == (Sq // B) * S
+    for W in (3, 4):
+        mc, mi, fc, fi, pairs = c_oracle.block_index(4352, 4608, C, S, W, 256)
+        want = ka["configs"]["cfg0"][f"W{W}"]
+        assert (int(mc.sum()), int(fc.sum()), pairs, int((mc + fc).max())) == \
+            (want["partial"], want["full"], want["pairs"], want["max_tiles_per_row_tile"])
