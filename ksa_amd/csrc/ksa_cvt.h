@@ -24,6 +24,25 @@ struct KsaCvt<KsaBf16> {
     static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
         return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), c, false);
     }
+    // Two / four such products with a zero addend.  The compiler only has the accumulating
+    // two-operand form for a zero addend and clears its register first; the three-operand form
+    // with an inline zero is written out here.  The wait states at the end cover a result read
+    // by the next vector instruction (3 wait states, DOT -> VALU): the compiler's hazard handling
+    // does not look inside an assembly statement.
+    static __device__ __forceinline__ void dot2z_x2(uint32_t a0, uint32_t b0, uint32_t a1, uint32_t b1,
+                                                    float& r0, float& r1) {
+        asm("v_dot2_f32_bf16 %0, %2, %3, 0\n\tv_dot2_f32_bf16 %1, %4, %5, 0\n\ts_nop 2"
+            : "=&v"(r0), "=&v"(r1)
+            : "v"(a0), "v"(b0), "v"(a1), "v"(b1));
+    }
+    static __device__ __forceinline__ void dot2z_x4(uint32_t a0, uint32_t b0, uint32_t a1, uint32_t b1,
+                                                    uint32_t a2, uint32_t b2, uint32_t a3, uint32_t b3,
+                                                    float& r0, float& r1, float& r2, float& r3) {
+        asm("v_dot2_f32_bf16 %0, %4, %5, 0\n\tv_dot2_f32_bf16 %1, %6, %7, 0\n\t"
+            "v_dot2_f32_bf16 %2, %8, %9, 0\n\tv_dot2_f32_bf16 %3, %10, %11, 0\n\ts_nop 2"
+            : "=&v"(r0), "=&v"(r1), "=&v"(r2), "=&v"(r3)
+            : "v"(a0), "v"(b0), "v"(a1), "v"(b1), "v"(a2), "v"(b2), "v"(a3), "v"(b3));
+    }
     static constexpr uint32_t kOnes = 0x3f803f80u;  // (1.0, 1.0)
 };
 template <>
@@ -49,6 +68,15 @@ struct KsaCvt<KsaF16> {
     static __device__ __forceinline__ float hi(uint32_t w) { return up((uint16_t)(w >> 16)); }
     static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
         return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a), __builtin_bit_cast(f16x2, b), c, false);
+    }
+    static __device__ __forceinline__ void dot2z_x2(uint32_t a0, uint32_t b0, uint32_t a1, uint32_t b1,
+                                                    float& r0, float& r1) {
+        r0 = dot2(a0, b0, 0.f), r1 = dot2(a1, b1, 0.f);
+    }
+    static __device__ __forceinline__ void dot2z_x4(uint32_t a0, uint32_t b0, uint32_t a1, uint32_t b1,
+                                                    uint32_t a2, uint32_t b2, uint32_t a3, uint32_t b3,
+                                                    float& r0, float& r1, float& r2, float& r3) {
+        r0 = dot2(a0, b0, 0.f), r1 = dot2(a1, b1, 0.f), r2 = dot2(a2, b2, 0.f), r3 = dot2(a3, b3, 0.f);
     }
     static constexpr uint32_t kOnes = 0x3c003c00u;
 };

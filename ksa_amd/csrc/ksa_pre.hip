@@ -36,6 +36,7 @@ struct PreParams {
     int batch, S, Hq, Hkv;
     int tok_per_pass;  // tokens per workgroup pass: 4 / gcd(row groups per token, 4)
     float eps;
+    int passes_per_wg;  // passes of tok_per_pass consecutive tokens that one workgroup takes
 };
 
 template <typename T>
@@ -62,7 +63,7 @@ __device__ __forceinline__ float pre_row_sum(float ss) {
     return ss;
 }
 
-// One workgroup takes a few consecutive tokens at a time (grid-stride); its four waves share
+// One workgroup takes a few consecutive tokens; its four waves share
 // their head rows, RPW rows of one of q / k / v per wave instruction, the same number for every
 // wave.  Which tensor a wave instruction works on, the token's base addresses and the weights
 // are wave-uniform (scalar registers); a lane only adds its row's offset, so no index division
@@ -79,7 +80,6 @@ __global__ __launch_bounds__(256) void ksa_pre_attention_kernel(const PreParams 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int sub = lane / LPR;         // which of the wave's rows
     const int t = lane % LPR;           // 16-byte chunk inside the row
-    const int Hn[3] = {p.Hq, p.Hkv, p.Hkv};
     const int Gq = (p.Hq + RPW - 1) / RPW, Gk = (p.Hkv + RPW - 1) / RPW;
     const int G = Gq + 2 * Gk;
     const int ntok = p.batch * p.S;
@@ -109,78 +109,124 @@ __global__ __launch_bounds__(256) void ksa_pre_attention_kernel(const PreParams 
         ldst[w] = (uint32_t)sub * (uint32_t)p.d_hs[w] + 8 * t;
     }
 
-    // A workgroup pass covers TOK consecutive tokens, TOK * G row groups in all, a multiple of
-    // four, so that its four waves get the same number of groups (G = 6 with 32 + 8 + 8 heads of
-    // 128: two tokens, three groups per wave).  (token, group) advance by four per wave step.
+    // A pass covers TOK consecutive tokens, TOK * G row groups in all, a multiple of four, so
+    // that the four waves get the same number of groups (G = 12 with 32 + 8 + 8 heads of 128: one
+    // token, three groups per wave); a workgroup takes a few consecutive passes and ends.
+    // (token, group) advance by four per wave step.  A wave walks its groups as one sequence and
+    // requests the rows of the next group (and the rotary row, when the token changes) before
+    // it works on the current one, so two of its row requests are in flight.
     const int TOK = p.tok_per_pass;
-    const int gi0 = wave % G, tl0 = wave / G;
-    for (int t0 = blockIdx.x * TOK; t0 < ntok; t0 += gridDim.x * TOK) {
-        int cur = -1;
-        uint32_t clo[4], chi[4], slo[4], shi[4];
-        int b = 0, s = 0;
-        for (int gi = gi0, tl = tl0; tl < TOK; gi += 4) {
-            while (gi >= G) {
-                gi -= G;
-                ++tl;
+    const int span = p.passes_per_wg * TOK;  // consecutive tokens of one workgroup
+    int gi = wave % G, tl = wave / G, t0 = blockIdx.x * span;
+    const int t_end = min(ntok, t0 + span);
+    struct Group {
+        bool live;             // wave-uniform: there is such a group
+        int which, tok, h0;
+        const uint16_t* sbase;
+        uint16_t* dbase;
+    };
+    int nb = 0, ns = 0, ntk = -1;  // batch index and position of the token of the last group
+    auto next_group = [&]() {
+        Group g;
+        while (gi >= G) {
+            gi -= G;
+            ++tl;
+        }
+        if (tl >= TOK) {  // groups per wave and pass are equal, so tl < 2 * TOK here
+            tl -= TOK;
+            t0 += TOK;
+        }
+        g.tok = t0 + tl;
+        g.live = g.tok < t_end;  // tokens only grow along the sequence: the first miss ends it
+        if (g.live && g.tok != ntk) {
+            ntk = g.tok;
+            nb = g.tok / p.S;
+            ns = g.tok - nb * p.S;
+        }
+        g.which = gi < Gq ? 0 : (gi < Gq + Gk ? 1 : 2);
+        g.h0 = (gi - (g.which == 0 ? 0 : (g.which == 1 ? Gq : Gq + Gk))) * RPW;
+        g.sbase = p.src[g.which] + nb * p.s_bs[g.which] + (int64_t)ns * p.s_rs[g.which] + (int64_t)g.h0 * p.s_hs[g.which];
+        g.dbase = p.dst[g.which] + nb * p.d_bs[g.which] + (int64_t)ns * p.d_rs[g.which] + (int64_t)g.h0 * p.d_hs[g.which];
+        gi += 4;
+        return g;
+    };
+    auto pick = [](int which, const uint32_t (&a)[3]) { return which == 0 ? a[0] : (which == 1 ? a[1] : a[2]); };
+    // a lane group beyond the last head is idle as a whole, exchange partners included
+    auto lane_ok = [&](const Group& g) { return g.h0 + sub < (g.which == 0 ? p.Hq : p.Hkv); };
+    const u32x4 zero4 = {0u, 0u, 0u, 0u};
+
+    Group g = next_group();
+    u32x4 raw = zero4, craw = zero4, sraw = zero4;
+    if (g.live) {
+        craw = *reinterpret_cast<const u32x4*>(p.cos + nb * p.c_bs + (int64_t)ns * p.c_rs + 8 * t);
+        sraw = *reinterpret_cast<const u32x4*>(p.sin + nb * p.c_bs + (int64_t)ns * p.c_rs + 8 * t);
+        // every byte of q, k, v is touched once: non-temporal accesses
+        if (lane_ok(g)) raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(g.sbase + pick(g.which, lsrc)));
+    }
+    int cur = -1;  // token whose rotary row is split below
+    uint32_t clo[4], chi[4], slo[4], shi[4];
+    while (g.live) {
+        const Group n = next_group();
+        u32x4 raw_n = zero4, craw_n = craw, sraw_n = sraw;
+        if (n.live) {
+            if (n.tok != g.tok) {
+                craw_n = *reinterpret_cast<const u32x4*>(p.cos + nb * p.c_bs + (int64_t)ns * p.c_rs + 8 * t);
+                sraw_n = *reinterpret_cast<const u32x4*>(p.sin + nb * p.c_bs + (int64_t)ns * p.c_rs + 8 * t);
             }
-            const int tok = t0 + tl;
-            if (tl >= TOK || tok >= ntok) break;
-            if (tok != cur) {  // wave-uniform: the rotary row of this token, split like the weights
-                cur = tok;
-                b = tok / p.S;
-                s = tok - b * p.S;
-                const u32x4 craw = *reinterpret_cast<const u32x4*>(p.cos + b * p.c_bs + (int64_t)s * p.c_rs + 8 * t);
-                const u32x4 sraw = *reinterpret_cast<const u32x4*>(p.sin + b * p.c_bs + (int64_t)s * p.c_rs + 8 * t);
+            if (lane_ok(n)) raw_n = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(n.sbase + pick(n.which, lsrc)));
+        }
+        if (g.tok != cur) {  // wave-uniform: the rotary row of this token, split like the weights
+            cur = g.tok;
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {  // the sine carries the rotate_half sign
-                    clo[i] = craw[i] & 0xffffu;
-                    chi[i] = craw[i] & 0xffff0000u;
-                    slo[i] = (sraw[i] ^ sgn_bits) & 0xffffu;
-                    shi[i] = (sraw[i] ^ sgn_bits) & 0xffff0000u;
-                }
+            for (int i = 0; i < 4; ++i) {  // the sine carries the rotate_half sign
+                clo[i] = craw[i] & 0xffffu;
+                chi[i] = craw[i] & 0xffff0000u;
+                slo[i] = (sraw[i] ^ sgn_bits) & 0xffffu;
+                shi[i] = (sraw[i] ^ sgn_bits) & 0xffff0000u;
             }
-            const int which = gi < Gq ? 0 : (gi < Gq + Gk ? 1 : 2);          // wave-uniform
-            const int h0 = (gi - (which == 0 ? 0 : (which == 1 ? Gq : Gq + Gk))) * RPW;
-            const uint16_t* sbase = p.src[which] + b * p.s_bs[which] + (int64_t)s * p.s_rs[which] + (int64_t)h0 * p.s_hs[which];
-            uint16_t* dbase = p.dst[which] + b * p.d_bs[which] + (int64_t)s * p.d_rs[which] + (int64_t)h0 * p.d_hs[which];
-            if (h0 + sub >= Hn[which]) continue;  // a whole lane group is idle: its exchange partners are idle too
-            // every byte is touched once: non-temporal accesses
-            const u32x4 raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(sbase + lsrc[which]));
-            uint16_t* dp = dbase + ldst[which];
-            if (which == 2) {  // v: layout change only
+        }
+        if (lane_ok(g)) {
+            uint16_t* dp = g.dbase + pick(g.which, ldst);
+            if (g.which == 2) {  // v: layout change only
                 __builtin_nontemporal_store(raw, reinterpret_cast<u32x4*>(dp));
-                continue;
-            }
-            float ss = 0.f;
+            } else {
+                float ss = 0.f;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) ss = C::dot2(raw[i], raw[i], ss);
-            ss = pre_row_sum<LPR>(ss);
-            const float inv = rsqrtf(ss * (1.0f / D) + p.eps);
-            // z = round(w * round(x * inv)), kept packed for the exchange
-            u32x4 zp;
-            auto scale_rows = [&](const uint32_t (&wl)[4], const uint32_t (&wh)[4]) {
+                for (int i = 0; i < 4; ++i) ss = C::dot2(raw[i], raw[i], ss);
+                ss = pre_row_sum<LPR>(ss);
+                const float inv = rsqrtf(ss * (1.0f / D) + p.eps);
+                // z = round(w * round(x * inv)), kept packed for the exchange
+                u32x4 zp;
+                auto scale_rows = [&](const uint32_t (&wl)[4], const uint32_t (&wh)[4]) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const uint32_t y = C::down2(C::lo(raw[i]) * inv, C::hi(raw[i]) * inv);
+                        float z0, z1;
+                        C::dot2z_x2(y, wl[i], y, wh[i], z0, z1);
+                        zp[i] = C::down2(z0, z1);
+                    }
+                };
+                if (g.which == 0) scale_rows(wlo[0], whi[0]);
+                else scale_rows(wlo[1], whi[1]);
+                // out = round(round(z cos) + round(rot(z) sin)); the two rounded terms of an
+                // element are packed together and added by a dot product with (1, 1)
+                u32x4 outp;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    const uint32_t y = C::down2(C::lo(raw[i]) * inv, C::hi(raw[i]) * inv);
-                    zp[i] = C::down2(C::dot2(y, wl[i], 0.f), C::dot2(y, wh[i], 0.f));
+                    uint32_t pp;  // the partner half of the row
+                    if constexpr (LPR == 16) pp = pre_row_ror<8>(zp[i]);
+                    else pp = (uint32_t)__shfl_xor((int)zp[i], LPR / 2);
+                    float c0, s0, c1, s1, o0, o1;
+                    C::dot2z_x4(zp[i], clo[i], pp, slo[i], zp[i], chi[i], pp, shi[i], c0, s0, c1, s1);
+                    const uint32_t e0 = C::down2(c0, s0), e1 = C::down2(c1, s1);
+                    C::dot2z_x2(e0, C::kOnes, e1, C::kOnes, o0, o1);
+                    outp[i] = C::down2(o0, o1);
                 }
-            };
-            if (which == 0) scale_rows(wlo[0], whi[0]);
-            else scale_rows(wlo[1], whi[1]);
-            // out = round(round(z cos) + round(rot(z) sin)); the two rounded terms of an element
-            // are packed together and added by a dot product with (1, 1)
-            u32x4 outp;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                uint32_t pp;  // the partner half of the row
-                if constexpr (LPR == 16) pp = pre_row_ror<8>(zp[i]);
-                else pp = (uint32_t)__shfl_xor((int)zp[i], LPR / 2);
-                const uint32_t e0 = C::down2(C::dot2(zp[i], clo[i], 0.f), C::dot2(pp, slo[i], 0.f));
-                const uint32_t e1 = C::down2(C::dot2(zp[i], chi[i], 0.f), C::dot2(pp, shi[i], 0.f));
-                outp[i] = C::down2(C::dot2(e0, C::kOnes, 0.f), C::dot2(e1, C::kOnes, 0.f));
+                __builtin_nontemporal_store(outp, reinterpret_cast<u32x4*>(dp));
             }
-            __builtin_nontemporal_store(outp, reinterpret_cast<u32x4*>(dp));
         }
+        g = n;
+        raw = raw_n, craw = craw_n, sraw = sraw_n;
     }
 }
 
@@ -189,9 +235,13 @@ int launch_pre(PreParams p, hipStream_t stream) {
     constexpr int RPW = 64 / (D / 8);
     const int G = (p.Hq + RPW - 1) / RPW + 2 * ((p.Hkv + RPW - 1) / RPW);
     p.tok_per_pass = (G % 4 == 0) ? 1 : (G % 2 == 0 ? 2 : 4);
-    int64_t blocks = ((int64_t)p.batch * p.S + p.tok_per_pass - 1) / p.tok_per_pass;
-    const int64_t cap = 256 * 16;                        // grid-stride beyond that
-    if (blocks > cap) blocks = cap;
+    // Short-lived workgroups over consecutive tokens, in launch order, keep the window of
+    // addresses in flight narrow: measured 5 % faster than a grid-stride loop of long-lived
+    // workgroups over the same accesses (a plain copy shows the same preference, 6.2 against
+    // 4.9 TB/s).  Four passes amortise a workgroup's set-up; 2 .. 8 measure alike.
+    p.passes_per_wg = 4;
+    const int64_t span = (int64_t)p.passes_per_wg * p.tok_per_pass;
+    const int64_t blocks = ((int64_t)p.batch * p.S + span - 1) / span;
     hipLaunchKernelGGL((ksa_pre_attention_kernel<T, D>), dim3((unsigned)blocks), dim3(256), 0, stream, p);
     return ksa_check_launch();
 }
@@ -211,7 +261,7 @@ extern "C" int ksa_pre_attention(const void* q, const void* k, const void* v, co
         !cos_strides)
         return KSA_ERR_NULL;
     if (batch <= 0 || S <= 0 || Hq <= 0 || Hkv <= 0 || !(eps >= 0.f)) return KSA_ERR_INVALID;
-    if ((int64_t)batch * S >= (1ll << 31)) return KSA_ERR_INVALID;
+    if ((int64_t)batch * S >= (1ll << 31) - 64) return KSA_ERR_INVALID;  // token indices, plus a workgroup's span, in 32 bits
     // a lane's row offset inside one wave instruction (at most 8 head rows) is kept in 32 bits
     for (const int64_t* s3 : {q_strides, k_strides, v_strides, q_out_strides, k_out_strides, v_out_strides})
         if (s3[2] < 0 || s3[2] * 8 + 128 >= (1ll << 32)) return KSA_ERR_INVALID;
