@@ -77,11 +77,12 @@ def test_index_cfg2_known_answer():
     assert int((idx[0] + idx[2]).max()) == 139
 
 
-@pytest.fixture(params=[None, "32", "64"], ids=["default", "rows32", "rows64"])
+@pytest.fixture(params=["0", "32", "64", None], ids=["two_heads", "rows32", "rows64", "auto"])
 def wave_rows(request, monkeypatch):
     """The workgroup shapes of the prefill kernel (D = 128, even group size): two heads on 8
-    waves (default), one head on 4 waves (KSA_PREFILL_ROWS_PER_WAVE=32) and two heads on 4
-    waves with 64 query rows per wave (=64).  The library reads the variable on every call."""
+    waves (KSA_PREFILL_ROWS_PER_WAVE=0; what a long launch gets by default), one head on 4 waves
+    (=32; what a short launch gets by default) and two heads on 4 waves with 64 query rows per
+    wave (=64); unset = the library's own choice.  The library reads the variable on every call."""
     if request.param is None:
         monkeypatch.delenv("KSA_PREFILL_ROWS_PER_WAVE", raising=False)
     else:
@@ -389,7 +390,7 @@ def test_prefill_random_shapes(seed, monkeypatch):
         mode = str(rng.choice(["prefix", "prefix", "inline", "physical"]))
         skip = bool(rng.integers(0, 2))
         dtype = torch.bfloat16 if rng.integers(0, 4) else torch.float16
-        shape = str(rng.choice(["", "32", "64"]))
+        shape = str(rng.choice(["", "0", "32", "64"]))
         if shape:
             monkeypatch.setenv("KSA_PREFILL_ROWS_PER_WAVE", shape)
         else:
