@@ -794,11 +794,11 @@ extern "C" int ksa_prefill_fwd(const void* q, const void* k, const void* v, void
     // Workgroup shape (D = 128, even group size; anything else uses one head per workgroup):
     // default two heads on 8 waves; KSA_PREFILL_ROWS_PER_WAVE=32 (or a short launch) one head on 4 waves;
     // =64 two heads on 4 waves with 64 query rows per wave (one wave per SIMD).
-    // A short launch (fewer than 8 two-head workgroups per CU of the 256) takes the one-head shape:
+    // A short launch (fewer than 16 two-head workgroups per CU of the 256) takes the one-head shape:
     // two of its workgroups share a CU and hide each other's start and end (8k rows: +9 %,
-    // 32k rows and up: the same within 1 %).
+    // 16k: +4 %, 24k: +1.5 %, 32k rows and up: the same within 1 %).
     const char* rpw = getenv("KSA_PREFILL_ROWS_PER_WAVE");
-    p.shape = rpw ? atoi(rpw) : ((int64_t)p.M * (Hq / 2) * batch < 8 * 256 ? 32 : 0);
+    p.shape = rpw ? atoi(rpw) : ((int64_t)p.M * (Hq / 2) * batch < 16 * 256 ? 32 : 0);
 
     hipStream_t st = (hipStream_t)stream;
     if (dtype == KSA_DTYPE_BF16) {
