@@ -182,3 +182,23 @@ def test_cache_summary_growth():
     a, b = model.attention_range()
     assert cache.attention_range(0) == (a, b)
     assert cache.key_cache[0][0, 0, a:b, 0].float().tolist() == [float(x) for x in model.buf[a:b]]
+
+
+def test_split_heuristics_are_host_only_and_bounded():
+    """`ksa_gemm_rows_auto_splits` / `ksa_decode_auto_splits` run on the host: the decoder's
+    shapes get the split counts the kernels were tuned with, and any shape gets a count the
+    kernels accept (at least 1, at most 16, never a slice shorter than one 512-element chunk)."""
+    from ksa_amd import _lib
+    L = _lib.lib()
+    known = {(6144, 2560): 5, (2560, 4096): 8, (19456, 2560): 5, (2560, 9728): 13, (151936, 2560): 1}
+    for (N, K), want in known.items():
+        assert L.ksa_gemm_rows_auto_splits(N, K) == want, (N, K)
+    rng = np.random.default_rng(0)
+    for _ in range(200):
+        N, K = int(rng.integers(1, 200000)), 32 * int(rng.integers(1, 600))
+        sp = L.ksa_gemm_rows_auto_splits(N, K)
+        assert 1 <= sp <= 16 and sp <= max(1, K // 512), (N, K, sp)
+        assert L.ksa_gemm_rows_workspace_bytes(N, sp) == (0 if sp == 1 else sp * 16 * N * 4)
+    for b, h, rows in [(64, 8, 17288), (8, 8, 40000), (1, 1, 100), (1, 8, 1 << 20)]:
+        assert 1 <= L.ksa_decode_auto_splits(b, h, rows) <= 64
+    assert L.ksa_decode_auto_splits(64, 8, 17288) == 1
