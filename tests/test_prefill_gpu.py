@@ -53,28 +53,40 @@ def test_index_odd_shapes(case, skip_old):
     _index_case(Sq, C, S, W, P, skip_old, tm, tn)
 
 
+def _known_answers(cfg):
+    """tests/golden/known_answers.json: tile totals derived independently of oracle and kernel."""
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(__file__), "golden", "known_answers.json")) as f:
+        ka = json.load(f)
+    assert (ka["C"], ka["S"], ka["tile_m"], ka["tile_n"]) == (128, 8, 128, 64)
+    return ka["configs"][cfg]
+
+
 def test_index_cfg1_known_answer():
-    """cfg 1 (256 chunks): totals derived independently of both oracle and kernel."""
+    """cfg 1 (256 chunks): totals of the golden fixture."""
     import ksa_amd
-    for W, (npart, nfull) in {3: (6558, 430), 4: (7076, 445)}.items():
-        idx = ksa_amd.compute_block_sparsity(34816, 36864, 128, 8, W)
-        assert int(idx[0].sum()) == npart and int(idx[2].sum()) == nfull
+    ka = _known_answers("cfg1")
+    for W in (3, 4):
+        idx = ksa_amd.compute_block_sparsity(ka["Sq"], ka["Sq"] + ka["P"], 128, 8, W)
+        assert int(idx[0].sum()) == ka[f"W{W}"]["partial"] and int(idx[2].sum()) == ka[f"W{W}"]["full"]
     _index_case(34816, 128, 8, 4, 2048, False)
 
 
 def test_index_cfg2_known_answer():
     """cfg 2 (1024 chunks, 128k): tile totals and the max tiles of one row tile."""
     import ksa_amd
-    for W, (npart, nfull) in {3: (75438, 4798), 4: (77540, 4861)}.items():
-        idx = ksa_amd.compute_block_sparsity(139264, 147456, 128, 8, W)
-        assert int(idx[0].sum()) == npart and int(idx[2].sum()) == nfull
+    ka = _known_answers("cfg2")
+    for W in (3, 4):
+        idx = ksa_amd.compute_block_sparsity(ka["Sq"], ka["Sq"] + ka["P"], 128, 8, W)
+        assert int(idx[0].sum()) == ka[f"W{W}"]["partial"] and int(idx[2].sum()) == ka[f"W{W}"]["full"]
         # ascending lists, zero tails
         mi = idx[1][0, 0]
         cnt = idx[0][0, 0]
         ar = torch.arange(mi.shape[1], device=mi.device)[None, :]
         assert bool((mi[:, 1:] > mi[:, :-1])[ar[:, 1:] < cnt[:, None]].all())
         assert int(mi[ar >= cnt[:, None]].abs().sum()) == 0
-    assert int((idx[0] + idx[2]).max()) == 139
+    assert int((idx[0] + idx[2]).max()) == ka["W4"]["max_tiles_per_row_tile"]
 
 
 @pytest.fixture(params=["0", "32", "64", None], ids=["two_heads", "rows32", "rows64", "auto"])
