@@ -42,7 +42,10 @@ __global__ __launch_bounds__(kIdxThreads) void ksa_block_index_kernel(
             const int32_t b = ksa_imin(mk.Sk, a + tile_n);
             const int32_t width = b - a;
             bool any_vis = false, any_hid = false;
-            for (int q = q0; q < q1; ++q) {
+            // every rule is causal in the key's sequence position (column - P): a tile that
+            // starts behind the last row of the m-tile is empty, no rows to look at
+            const int q_end = a >= mk.P + q1 ? q0 : q1;
+            for (int q = q0; q < q_end; ++q) {
                 const int32_t cnt = ksa_count_visible(mk, q, a, b);
                 any_vis |= cnt > 0;
                 any_hid |= cnt < width;
