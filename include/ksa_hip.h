@@ -113,14 +113,18 @@ int ksa_copy_rows(const void* src, void* dst, const int32_t* src_index,
  *   q_weight, k_weight [D]; cos, sin [batch or 1, S, D] with cos_strides {batch, row}
  *   q_out, k_out, v_out: any {batch, row, head} strides -- the [batch, S, H, D] layout of
  *   ksa_prefill_fwd, or rows of a [batch, H, capacity, D] cache tensor (pointer at the
- *   first destination row).  q_out may alias q, k_out k, v_out v (same strides). */
+ *   first destination row).  q_out may alias q, k_out k, v_out v (same strides).
+ *   kv_out_row_seq: NULL, or int32 [batch] in device memory: sequence b's k and v go
+ *   kv_out_row_seq[b] rows (of k_out_strides[1] / v_out_strides[1]) further down - the cache
+ *   cursor of update_text (HF:306-336) when only the device knows it (graph replay); the
+ *   caller guarantees the rows exist. */
 int ksa_pre_attention(const void* q, const void* k, const void* v, const void* q_weight,
                       const void* k_weight, const void* cos, const void* sin, void* q_out,
                       void* k_out, void* v_out, int batch, int S, int Hq, int Hkv, int D, int dtype,
                       const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
                       const int64_t* q_out_strides, const int64_t* k_out_strides,
-                      const int64_t* v_out_strides, const int64_t* cos_strides, float eps,
-                      void* stream);
+                      const int64_t* v_out_strides, const int64_t* cos_strides,
+                      const int32_t* kv_out_row_seq, float eps, void* stream);
 
 /* Residual add + RMSNorm over the hidden size, one pass.
  * Replaces Qwen3RMSNorm.forward (HF:64-79: fp32 normalisation, rounded to the 16-bit type, times

@@ -29,7 +29,7 @@ _SIGNATURES = {
     "ksa_decode_fwd": (_int, [_vp] * 6 + [_int] * 8 + [_i64p] * 4
                        + [ctypes.c_float, _int, _vp, ctypes.c_size_t, _vp]),
     "ksa_copy_rows": (_int, [_vp] * 4 + [_int] * 6 + [_i64p] * 2 + [_vp]),
-    "ksa_pre_attention": (_int, [_vp] * 10 + [_int] * 6 + [_i64p] * 7 + [ctypes.c_float, _vp]),
+    "ksa_pre_attention": (_int, [_vp] * 10 + [_int] * 6 + [_i64p] * 7 + [_vp, ctypes.c_float, _vp]),
     "ksa_add_rmsnorm": (_int, [_vp] * 5 + [ctypes.c_longlong, _int] + [ctypes.c_longlong] * 4
                         + [_int, ctypes.c_float, _vp]),
     "ksa_silu_mul": (_int, [_vp] * 3 + [ctypes.c_longlong, _int] + [ctypes.c_longlong] * 3 + [_int, _vp]),

@@ -28,6 +28,7 @@ struct PreParams {
     const uint16_t* src[3];   // q, k, v projections  [batch, S, H, D] by strides
     uint16_t* dst[3];         // q, k, v outputs
     const uint16_t* w[2];     // q_norm, k_norm weights [D]
+    const int32_t* kv_row;    // [batch] or null: row added to the k / v destination of a sequence
     const uint16_t* cos;      // [batch or 1, S, D]
     const uint16_t* sin;
     int64_t s_bs[3], s_rs[3], s_hs[3];
@@ -146,7 +147,9 @@ __global__ __launch_bounds__(256) void ksa_pre_attention_kernel(const PreParams 
         g.which = gi < Gq ? 0 : (gi < Gq + Gk ? 1 : 2);
         g.h0 = (gi - (g.which == 0 ? 0 : (g.which == 1 ? Gq : Gq + Gk))) * RPW;
         g.sbase = p.src[g.which] + nb * p.s_bs[g.which] + (int64_t)ns * p.s_rs[g.which] + (int64_t)g.h0 * p.s_hs[g.which];
-        g.dbase = p.dst[g.which] + nb * p.d_bs[g.which] + (int64_t)ns * p.d_rs[g.which] + (int64_t)g.h0 * p.d_hs[g.which];
+        // (k and v may go to a row of their sequence that the host does not know: a cache cursor)
+        const int64_t drow = ns + ((g.which != 0 && p.kv_row) ? p.kv_row[nb] : 0);
+        g.dbase = p.dst[g.which] + nb * p.d_bs[g.which] + drow * p.d_rs[g.which] + (int64_t)g.h0 * p.d_hs[g.which];
         gi += 4;
         return g;
     };
@@ -254,7 +257,8 @@ extern "C" int ksa_pre_attention(const void* q, const void* k, const void* v, co
                                  int dtype, const int64_t* q_strides, const int64_t* k_strides,
                                  const int64_t* v_strides, const int64_t* q_out_strides,
                                  const int64_t* k_out_strides, const int64_t* v_out_strides,
-                                 const int64_t* cos_strides, float eps, void* stream) {
+                                 const int64_t* cos_strides, const int32_t* kv_out_row_seq, float eps,
+                                 void* stream) {
     if (!q || !k || !v || !q_weight || !k_weight || !cos || !sin || !q_out || !k_out || !v_out)
         return KSA_ERR_NULL;
     if (!q_strides || !k_strides || !v_strides || !q_out_strides || !k_out_strides || !v_out_strides ||
@@ -281,6 +285,7 @@ extern "C" int ksa_pre_attention(const void* q, const void* k, const void* v, co
     p.dst[0] = (uint16_t*)q_out, p.dst[1] = (uint16_t*)k_out, p.dst[2] = (uint16_t*)v_out;
     p.w[0] = (const uint16_t*)q_weight, p.w[1] = (const uint16_t*)k_weight;
     p.cos = (const uint16_t*)cos, p.sin = (const uint16_t*)sin;
+    p.kv_row = kv_out_row_seq;
     const int64_t* in[] = {q_strides, k_strides, v_strides};
     const int64_t* out[] = {q_out_strides, k_out_strides, v_out_strides};
     for (int i = 0; i < 3; ++i) {

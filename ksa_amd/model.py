@@ -360,9 +360,11 @@ class KsaQwen3ForCausalLM:
             kind = 1 if cache.is_large_window[li] else 0
             x, h = self._add_norm(delta, x, lw["input_layernorm"])
             q, k, v = self._qkv(lw, h, None)
-            q, k, v = ops.pre_attention(q, k, v, lw["q_norm"], lw["k_norm"], cos, sin, cfg.rms_norm_eps)
-            cache._move_rows(k.transpose(1, 2), cache.key_cache[li], 1, dst_start_seq=st["cur"][kind, 0])
-            cache._move_rows(v.transpose(1, 2), cache.value_cache[li], 1, dst_start_seq=st["cur"][kind, 0])
+            # k and v go straight to the cache row the device-side cursor names
+            q, _, _ = ops.pre_attention(q, k, v, lw["q_norm"], lw["k_norm"], cos, sin, cfg.rms_norm_eps,
+                                        k_out=cache.key_cache[li][:, :, :1].transpose(1, 2),
+                                        v_out=cache.value_cache[li][:, :, :1].transpose(1, 2),
+                                        kv_out_row=st["cur"][kind, 0])
             attn = ops.decode(q.transpose(1, 2), cache.key_cache[li], cache.value_cache[li],
                               st["cur"][kind, 1], st["cur"][kind, 2], self.scaling)
             x, h = self._add_norm(ops.linear(attn.reshape(b, 1, -1), lw["o_proj"]), x, lw["post_attention_layernorm"])

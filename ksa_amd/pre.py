@@ -25,14 +25,17 @@ def _bsh(t):  # element strides of a [batch, rows, heads, D] view
 def pre_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q_norm_weight: torch.Tensor,
                   k_norm_weight: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, eps: float = 1e-6,
                   q_out: Optional[torch.Tensor] = None, k_out: Optional[torch.Tensor] = None,
-                  v_out: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+                  v_out: Optional[torch.Tensor] = None,
+                  kv_out_row: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """q [b, S, Hq, D], k, v [b, S, Hkv, D] (views of the projection outputs, head_dim contiguous);
     cos, sin [b or 1, S, D] as returned by the rotary embedding module, in the dtype of q.
 
     Returns (q', k', v) with q' = rope(q_norm(q)), k' = rope(k_norm(k)) in [b, S, H, D].  `*_out`
     may be given as [b, S, H, D]-shaped views with arbitrary batch/row/head strides, e.g.
     `cache_k[:, :, start:start + S].transpose(1, 2)` to write the keys straight into a
-    [b, Hkv, capacity, D] cache tensor; they may alias the inputs.
+    [b, Hkv, capacity, D] cache tensor; they may alias the inputs.  `kv_out_row` (int32 [b] on
+    the GPU) moves sequence b's k and v `kv_out_row[b]` rows further down their outputs: the
+    cache cursor when only the device knows it (a recorded step that is replayed).
     """
     assert q.dtype in _DT and k.dtype == q.dtype and v.dtype == q.dtype, "q, k, v must share bf16 or fp16"
     assert q.is_cuda and k.is_cuda and v.is_cuda, "inputs must be on a GPU"
@@ -55,12 +58,17 @@ def pre_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q_norm_weig
         assert given.shape == like.shape and given.dtype == like.dtype and given.stride(3) == 1
         outs.append(given)
     qo, ko, vo = outs
+    if kv_out_row is not None:
+        assert kv_out_row.is_cuda and kv_out_row.dtype == torch.int32 and kv_out_row.shape == (b,) \
+            and kv_out_row.is_contiguous(), "kv_out_row must be a contiguous int32 [b] GPU tensor"
+        assert k_out is not None and v_out is not None, "kv_out_row needs k_out and v_out"
     cstr = (ctypes.c_int64 * 3)(cos.stride(0) if cos.shape[0] > 1 else 0, cos.stride(1), 0)
     L = _lib.lib()
     with torch.cuda.device(q.device):
         rc = L.ksa_pre_attention(q.data_ptr(), k.data_ptr(), v.data_ptr(), qw.data_ptr(), kw.data_ptr(),
                                  cos.data_ptr(), sin.data_ptr(), qo.data_ptr(), ko.data_ptr(), vo.data_ptr(),
                                  b, S, Hq, Hkv, D, _DT[q.dtype], _bsh(q), _bsh(k), _bsh(v), _bsh(qo),
-                                 _bsh(ko), _bsh(vo), cstr, float(eps), _lib.stream_ptr(q.device))
+                                 _bsh(ko), _bsh(vo), cstr, None if kv_out_row is None else kv_out_row.data_ptr(),
+                                 float(eps), _lib.stream_ptr(q.device))
     _lib.check(rc, "ksa_pre_attention")
     return qo, ko, vo

@@ -34,7 +34,8 @@ class OracleOps:
         self.cache_cls = HostCache
 
     @staticmethod
-    def pre_attention(q, k, v, qw, kw, cos, sin, eps, q_out=None, k_out=None, v_out=None):
+    def pre_attention(q, k, v, qw, kw, cos, sin, eps, q_out=None, k_out=None, v_out=None, kv_out_row=None):
+        assert kv_out_row is None, "device-side cache cursors belong to the GPU operators"
         qo, ko, vo = cpu_path.pre_attention(q, k, v, qw, kw, cos, sin, eps)
         res = []
         for given, val in ((q_out, qo), (k_out, ko), (v_out, vo)):

@@ -150,6 +150,41 @@ def test_pre_attention_gpu_writes_into_cache_layout_and_in_place():
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("S", [1, 3])
+def test_pre_attention_gpu_cache_row_from_device_memory(S):
+    """`kv_out_row`: each sequence's k and v land at the cache row a device-side int32 names
+    (the cursor of a recorded decode step), with the values of a call that was given the row on
+    the host; q and the rest of the cache are untouched by it."""
+    import ksa_amd
+    b, Hq, Hkv, D, dtype = 3, 8, 2, 128, torch.bfloat16
+    q, k, v, qw, kw = _inputs(b, S, Hq, Hkv, D, 9, dtype)
+    cos, sin, _ = _rope_tables(S, D, dtype=dtype)
+    dev = torch.device("cuda")
+    cap = 64
+    rows = [5, 40, 17]
+    args = [t.to(dev) for t in (q, k, v, qw, kw, cos, sin)]
+    kc = torch.zeros(b, Hkv, cap, D, dtype=dtype, device=dev)
+    vc = torch.zeros_like(kc)
+    cursor = torch.tensor(rows, dtype=torch.int32, device=dev)
+    q1, _, _ = ksa_amd.pre_attention(*args, eps=1e-6, k_out=kc[:, :, :S].transpose(1, 2),
+                                     v_out=vc[:, :, :S].transpose(1, 2), kv_out_row=cursor)
+    q0, k0, v0 = ksa_amd.pre_attention(*args, eps=1e-6)
+    torch.cuda.synchronize()
+    assert torch.equal(q0, q1)
+    for i, r in enumerate(rows):
+        assert torch.equal(kc[i, :, r:r + S].transpose(0, 1), k0[i])
+        assert torch.equal(vc[i, :, r:r + S].transpose(0, 1), v0[i])
+        kc[i, :, r:r + S] = 0
+        vc[i, :, r:r + S] = 0
+    assert kc.abs().max() == 0 and vc.abs().max() == 0
+    with pytest.raises(AssertionError):
+        ksa_amd.pre_attention(*args, eps=1e-6, kv_out_row=cursor)          # needs k_out / v_out
+    with pytest.raises(AssertionError):
+        ksa_amd.pre_attention(*args, eps=1e-6, k_out=kc[:, :, :S].transpose(1, 2),
+                              v_out=vc[:, :, :S].transpose(1, 2), kv_out_row=cursor.long())
+
+
+@pytest.mark.gpu
 def test_pre_attention_rejects_bad_inputs():
     import ksa_amd
     dev = torch.device("cuda")
