@@ -138,6 +138,18 @@ int ksa_add_rmsnorm(const void* x, const void* residual, const void* weight, voi
                     long long residual_row_stride, long long norm_row_stride,
                     long long sum_row_stride, int dtype, float eps, void* stream);
 
+/* ksa_add_rmsnorm whose x is not a tensor yet but the K-split partial sums that ksa_gemm_rows
+ * leaves in its workspace when called with out == NULL (fp32 [ksplit][16][H]): x = the sum over
+ * the splits in split order, rounded to the 16-bit type.  out_sum is bit-identical to
+ * ksa_gemm_rows with an output followed by ksa_add_rmsnorm; out_norm agrees to one unit in the
+ * last place (the mean square is summed in a different order).  One launch less per o_proj /
+ * down_proj -> residual add + norm (HF:944-952).  rows <= 16, H <= 8192; residual and out_sum
+ * are required. */
+int ksa_add_rmsnorm_partials(const float* partials, int ksplit, const void* residual,
+                             const void* weight, void* out_norm, void* out_sum, int rows, int H,
+                             long long residual_row_stride, long long norm_row_stride,
+                             long long sum_row_stride, int dtype, float eps, void* stream);
+
 /* out = round(SiLU(gate)) * up, the MLP activation of HF:507-514 (act_fn(gate_proj(x)) *
  * up_proj(x)) in one pass; gate and up may be the two halves of one fused projection output
  * (row strides in elements, multiples of 8; I a multiple of 8; rows < 2^31). */
@@ -151,7 +163,9 @@ int ksa_silu_mul(const void* gate, const void* up, void* out, long long rows, in
  *   x [M, K], w [N, K], out [M, N], 16-bit, row strides in elements (x, w: multiples of 8);
  *   K a multiple of 32; fp32 accumulation, one rounding at the end.
  * ksplit > 1 splits K over workgroups (ksa_gemm_rows_auto_splits) and needs
- * ksa_gemm_rows_workspace_bytes(N, ksplit) bytes of device workspace. */
+ * ksa_gemm_rows_workspace_bytes(N, ksplit) bytes of device workspace.  With ksplit > 1 out may
+ * be NULL: the partial sums (fp32 [ksplit][16][N]) are then left in the workspace for a consumer
+ * that adds them itself (ksa_add_rmsnorm_partials). */
 int ksa_gemm_rows_auto_splits(int N, int K);
 size_t ksa_gemm_rows_workspace_bytes(int N, int ksplit);
 int ksa_gemm_rows(const void* x, const void* w, void* out, int M, int N, int K, long long x_row_stride,

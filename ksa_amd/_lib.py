@@ -32,6 +32,8 @@ _SIGNATURES = {
     "ksa_pre_attention": (_int, [_vp] * 10 + [_int] * 6 + [_i64p] * 7 + [_vp, ctypes.c_float, _vp]),
     "ksa_add_rmsnorm": (_int, [_vp] * 5 + [ctypes.c_longlong, _int] + [ctypes.c_longlong] * 4
                         + [_int, ctypes.c_float, _vp]),
+    "ksa_add_rmsnorm_partials": (_int, [_vp, _int] + [_vp] * 4 + [_int, _int] + [ctypes.c_longlong] * 3
+                                 + [_int, ctypes.c_float, _vp]),
     "ksa_silu_mul": (_int, [_vp] * 3 + [ctypes.c_longlong, _int] + [ctypes.c_longlong] * 3 + [_int, _vp]),
     "ksa_gemm_rows_auto_splits": (_int, [_int, _int]),
     "ksa_gemm_rows_workspace_bytes": (ctypes.c_size_t, [_int, _int]),

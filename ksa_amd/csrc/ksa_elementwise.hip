@@ -14,8 +14,12 @@
 
 namespace {
 
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
 struct NormParams {
     const uint16_t* x;
+    const float* part;     // partial-sum variant: x = rounded sum of `ksplit` fp32 slices [ksplit][16][H]
+    int ksplit;
     const uint16_t* res;   // may be null
     const uint16_t* w;
     uint16_t* out_norm;
@@ -76,6 +80,86 @@ __global__ __launch_bounds__(256) void ksa_add_rmsnorm_kernel(const NormParams p
             }
         }
     }
+}
+
+// The same step for the few rows of a decode step when x is still the K-split partial sums of
+// the GEMM that produced it (fp32 [ksplit][16][H], as ksa_gemm_rows leaves them): one workgroup
+// per row adds the slices in split order, rounds (which is what the GEMM's own reduction does),
+// adds the residual and normalises.  NJ = 16-byte items per thread.
+template <typename T, int NJ>
+__global__ __launch_bounds__(256) void ksa_add_rmsnorm_partials_kernel(const NormParams p) {
+    using C = KsaCvt<T>;
+    __shared__ float s_ss[4];
+    const int tid = threadIdx.x;
+    const int row = blockIdx.x;
+    const int items = p.H / 8;
+    u32x4 r[NJ];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        const int idx = tid + 256 * j;
+        if (idx < items) {
+            float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            for (int sp0 = 0; sp0 < p.ksplit; sp0 += 8) {  // eight slices requested together
+                f32x4 lo[8], hi[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int sp = min(sp0 + u, p.ksplit - 1);
+                    const float* src = p.part + ((int64_t)sp * 16 + row) * p.H + 8 * idx;
+                    lo[u] = *reinterpret_cast<const f32x4*>(src);
+                    hi[u] = *reinterpret_cast<const f32x4*>(src + 4);
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    if (sp0 + u < p.ksplit) {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) acc[i] += lo[u][i], acc[4 + i] += hi[u][i];
+                    }
+                }
+            }
+            const u32x4 q = *reinterpret_cast<const u32x4*>(p.res + (int64_t)row * p.rs + 8 * idx);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t x2 = C::down2(acc[2 * i], acc[2 * i + 1]);
+                r[j][i] = C::down2(C::lo(x2) + C::lo(q[i]), C::hi(x2) + C::hi(q[i]));
+                const float a = C::lo(r[j][i]), b = C::hi(r[j][i]);
+                ss = fmaf(a, a, ss);
+                ss = fmaf(b, b, ss);
+            }
+            *reinterpret_cast<u32x4*>(p.out_sum + (int64_t)row * p.ss + 8 * idx) = r[j];
+        }
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) ss += __shfl_xor(ss, m);
+    if ((tid & 63) == 0) s_ss[tid >> 6] = ss;
+    __syncthreads();
+    ss = (s_ss[0] + s_ss[1]) + (s_ss[2] + s_ss[3]);
+    const float inv = rsqrtf(ss / (float)p.H + p.eps);
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        const int idx = tid + 256 * j;
+        if (idx < items) {
+            const u32x4 wv = *reinterpret_cast<const u32x4*>(p.w + 8 * idx);
+            u32x4 o;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t y = C::down2(C::lo(r[j][i]) * inv, C::hi(r[j][i]) * inv);
+                o[i] = C::down2(C::lo(wv[i]) * C::lo(y), C::hi(wv[i]) * C::hi(y));
+            }
+            *reinterpret_cast<u32x4*>(p.out_norm + (int64_t)row * p.ns + 8 * idx) = o;
+        }
+    }
+}
+
+template <typename T>
+int dispatch_norm_partials(const NormParams& p, hipStream_t st) {
+    const int need = (p.H / 8 + 255) / 256;
+    const dim3 grid((unsigned)p.rows), block(256);
+    if (need <= 1) hipLaunchKernelGGL((ksa_add_rmsnorm_partials_kernel<T, 1>), grid, block, 0, st, p);
+    else if (need <= 2) hipLaunchKernelGGL((ksa_add_rmsnorm_partials_kernel<T, 2>), grid, block, 0, st, p);
+    else if (need <= 4) hipLaunchKernelGGL((ksa_add_rmsnorm_partials_kernel<T, 4>), grid, block, 0, st, p);
+    else return KSA_ERR_UNSUPPORTED;
+    return ksa_check_launch();
 }
 
 template <typename T, int NI>
@@ -155,6 +239,31 @@ extern "C" int ksa_add_rmsnorm(const void* x, const void* residual, const void* 
     p.eps = eps;
     return dtype == KSA_DTYPE_BF16 ? dispatch_norm<KsaBf16>(p, (hipStream_t)stream)
                                    : dispatch_norm<KsaF16>(p, (hipStream_t)stream);
+}
+
+extern "C" int ksa_add_rmsnorm_partials(const float* partials, int ksplit, const void* residual,
+                                        const void* weight, void* out_norm, void* out_sum, int rows, int H,
+                                        long long residual_row_stride, long long norm_row_stride,
+                                        long long sum_row_stride, int dtype, float eps, void* stream) {
+    if (!partials || !residual || !weight || !out_norm || !out_sum) return KSA_ERR_NULL;
+    if (rows <= 0 || rows > 16 || ksplit < 1 || ksplit > 64 || H <= 0 || H % 8 != 0 || !(eps >= 0.f))
+        return KSA_ERR_INVALID;
+    if (dtype != KSA_DTYPE_BF16 && dtype != KSA_DTYPE_F16) return KSA_ERR_UNSUPPORTED;
+    if (!al16(partials) || !al16(residual) || !al16(weight) || !al16(out_norm) || !al16(out_sum)) return KSA_ERR_ALIGN;
+    if (residual_row_stride % 8 || norm_row_stride % 8 || sum_row_stride % 8) return KSA_ERR_ALIGN;
+    NormParams p{};
+    p.part = partials;
+    p.ksplit = ksplit;
+    p.res = (const uint16_t*)residual;
+    p.w = (const uint16_t*)weight;
+    p.out_norm = (uint16_t*)out_norm;
+    p.out_sum = (uint16_t*)out_sum;
+    p.rows = rows;
+    p.rs = residual_row_stride, p.ns = norm_row_stride, p.ss = sum_row_stride;
+    p.H = H;
+    p.eps = eps;
+    return dtype == KSA_DTYPE_BF16 ? dispatch_norm_partials<KsaBf16>(p, (hipStream_t)stream)
+                                   : dispatch_norm_partials<KsaF16>(p, (hipStream_t)stream);
 }
 
 extern "C" int ksa_silu_mul(const void* gate, const void* up, void* out, long long rows, int I,

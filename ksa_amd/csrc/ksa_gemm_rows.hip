@@ -124,7 +124,7 @@ template <typename T>
 int launch_gemm(const GemmParams& p, hipStream_t st) {
     dim3 grid((p.N + 63) / 64, p.ksplit);
     hipLaunchKernelGGL(ksa_gemm_rows_kernel<T>, grid, dim3(256), 0, st, p);
-    if (p.ksplit > 1) {
+    if (p.ksplit > 1 && p.out) {
         const int64_t n = (int64_t)p.M * p.N;
         hipLaunchKernelGGL(ksa_gemm_rows_reduce_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, p);
     }
@@ -156,7 +156,8 @@ extern "C" size_t ksa_gemm_rows_workspace_bytes(int N, int ksplit) {
 extern "C" int ksa_gemm_rows(const void* x, const void* w, void* out, int M, int N, int K, long long x_row_stride,
                              long long w_row_stride, long long out_row_stride, int dtype, int ksplit,
                              void* workspace, size_t workspace_bytes, void* stream) {
-    if (!x || !w || !out) return KSA_ERR_NULL;
+    if (!x || !w) return KSA_ERR_NULL;
+    if (!out && ksplit <= 1) return KSA_ERR_NULL;  // out may be null only to leave the partial sums to the caller
     if (M <= 0 || M > 16 || N <= 0 || K <= 0 || K % 32 != 0 || ksplit < 1 || ksplit > 64) return KSA_ERR_INVALID;
     if (dtype != KSA_DTYPE_BF16 && dtype != KSA_DTYPE_F16) return KSA_ERR_UNSUPPORTED;
     if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w)) & 15) return KSA_ERR_ALIGN;

@@ -13,6 +13,7 @@ from typing import Optional, Tuple
 import torch
 
 from . import _lib
+from .gemm import SplitKPartials
 
 _DT = {torch.bfloat16: 0, torch.float16: 1}
 
@@ -27,9 +28,31 @@ def _rows2d(t: torch.Tensor) -> torch.Tensor:
         return t.reshape(-1, t.shape[-1])
 
 
+def _add_rmsnorm_partials(x: SplitKPartials, residual: torch.Tensor, weight: torch.Tensor, eps: float):
+    assert residual is not None and residual.is_cuda and residual.dtype == x.dtype and tuple(residual.shape) == x.shape
+    H = x.shape[-1]
+    r2 = _rows2d(residual)
+    assert r2.shape[0] == x.rows
+    w = weight.to(x.dtype).contiguous()
+    assert w.shape == (H,)
+    out = torch.empty(r2.shape, dtype=x.dtype, device=x.device)
+    s = torch.empty(r2.shape, dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().ksa_add_rmsnorm_partials(x.workspace.data_ptr(), x.ksplit, r2.data_ptr(), w.data_ptr(),
+                                                 out.data_ptr(), s.data_ptr(), x.rows, H, r2.stride(0),
+                                                 out.stride(0), s.stride(0), _DT[x.dtype], float(eps),
+                                                 _lib.stream_ptr(x.device))
+    _lib.check(rc, "ksa_add_rmsnorm_partials")
+    return s.view(x.shape), out.view(x.shape)
+
+
 def add_rmsnorm(x: torch.Tensor, residual: Optional[torch.Tensor], weight: torch.Tensor,
                 eps: float = 1e-6) -> Tuple[torch.Tensor, torch.Tensor]:
-    """Returns (s, weight * rmsnorm(s)) with s = x + residual (s is x itself when residual is None)."""
+    """Returns (s, weight * rmsnorm(s)) with s = x + residual (s is x itself when residual is None).
+    x may be the `SplitKPartials` of a deferred `linear_rows` (then residual is required): the
+    partial sums are added here, with the same result as the reduced product would give."""
+    if isinstance(x, SplitKPartials):
+        return _add_rmsnorm_partials(x, residual, weight, eps)
     assert x.is_cuda and x.dtype in _DT, "x must be a bf16/fp16 GPU tensor"
     H = x.shape[-1]
     x2 = _rows2d(x)

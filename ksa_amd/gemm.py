@@ -15,8 +15,22 @@ _DT = {torch.bfloat16: 0, torch.float16: 1}
 MAX_ROWS = 16
 
 
-def linear_rows(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
-    """x [..., K] with at most 16 rows in all, weight [N, K] -> [..., N]."""
+class SplitKPartials:
+    """Output of `linear_rows(..., defer=True)` when K was split over workgroups: the fp32 partial
+    sums [ksplit, 16, N] as the kernel left them, for a consumer that adds them itself
+    (`ksa_amd.add_rmsnorm`).  `shape` / `dtype` are those of the tensor it stands for."""
+
+    def __init__(self, workspace: torch.Tensor, ksplit: int, rows: int, shape, dtype):
+        self.workspace, self.ksplit, self.rows, self.shape, self.dtype = workspace, ksplit, rows, tuple(shape), dtype
+
+    @property
+    def device(self):
+        return self.workspace.device
+
+
+def linear_rows(x: torch.Tensor, weight: torch.Tensor, defer: bool = False):
+    """x [..., K] with at most 16 rows in all, weight [N, K] -> [..., N].  With `defer`, a product
+    whose K is split over workgroups comes back as `SplitKPartials` (no reduction launch)."""
     assert x.is_cuda and x.dtype in _DT and weight.dtype == x.dtype, "bf16/fp16 GPU tensors"
     K = x.shape[-1]
     N = weight.shape[0]
@@ -27,16 +41,19 @@ def linear_rows(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     M = x2.shape[0]
     assert 1 <= M <= MAX_ROWS, "linear_rows is for at most 16 rows"
     L = _lib.lib()
-    out = torch.empty(M, N, dtype=x.dtype, device=x.device)
     ks = L.ksa_gemm_rows_auto_splits(N, K)
+    defer = defer and ks > 1
+    out = None if defer else torch.empty(M, N, dtype=x.dtype, device=x.device)
     ws = None
     ws_bytes = 0
     if ks > 1:
         ws_bytes = L.ksa_gemm_rows_workspace_bytes(N, ks)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
     with torch.cuda.device(x.device):
-        rc = L.ksa_gemm_rows(x2.data_ptr(), weight.data_ptr(), out.data_ptr(), M, N, K, x2.stride(0),
-                             weight.stride(0), out.stride(0), _DT[x.dtype], ks,
+        rc = L.ksa_gemm_rows(x2.data_ptr(), weight.data_ptr(), None if defer else out.data_ptr(), M, N, K,
+                             x2.stride(0), weight.stride(0), N, _DT[x.dtype], ks,
                              ws.data_ptr() if ws is not None else None, ws_bytes, _lib.stream_ptr(x.device))
     _lib.check(rc, "ksa_gemm_rows")
+    if defer:
+        return SplitKPartials(ws, ks, M, (*x.shape[:-1], N), x.dtype)
     return out.view(*x.shape[:-1], N)

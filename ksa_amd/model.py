@@ -142,12 +142,13 @@ class HipOps:
     def decode(self, q, kbuf, vbuf, start, end, scale):
         return self._decode(q, kbuf, vbuf, start, end, scale=scale)
 
-    def linear(self, x, weight):
+    def linear(self, x, weight, defer=False):
         """x W^T: the weight-streaming kernel for the few rows of a decode step, the library
-        GEMM otherwise."""
+        GEMM otherwise.  `defer`: the caller hands the result to `add_rmsnorm` as it is, so a
+        product split over K may come back as its partial sums (one launch less)."""
         rows = x.numel() // x.shape[-1]
         if rows <= self._max_rows and x.shape[-1] % 32 == 0:
-            return self._linear_rows(x, weight)
+            return self._linear_rows(x, weight, defer=defer)
         return F.linear(x, weight)
 
 
@@ -258,10 +259,11 @@ class KsaQwen3ForCausalLM:
         v = qkv[..., (Hq + Hkv) * D:].view(b, L, Hkv, D)
         return q, k, v
 
-    def _mlp(self, lw, x):
+    def _mlp(self, lw, x, defer=False):
+        """`defer`: the result only goes to `_add_norm` (see `HipOps.linear`)."""
         gu = self.ops.linear(x, lw["gate_up_proj"])
         I = self.config.intermediate_size
-        return self.ops.linear(self.ops.silu_mul(gu[..., :I], gu[..., I:]), lw["down_proj"])
+        return self.ops.linear(self.ops.silu_mul(gu[..., :I], gu[..., I:]), lw["down_proj"], defer=defer)
 
     def _logits(self, x_last, delta_last):
         _, h = self._add_norm(delta_last, x_last, self.w["norm"])
@@ -340,10 +342,13 @@ class KsaQwen3ForCausalLM:
                 sum_out = ops.decode(qh[:, :, 1:], k_cs, v_cs, 0, k_cs.shape[2], self.scaling)
                 cache.update_summary(kh[:, :, 1:], vh[:, :, 1:], li)
                 attn = torch.cat([text_out, sum_out], dim=1)
-            x, h = self._add_norm(ops.linear(attn.reshape(b, ids.shape[1], -1), lw["o_proj"]), x,
-                                  lw["post_attention_layernorm"])
-            delta = self._mlp(lw, h)
+            # a text step hands both products straight to the next norm; a boundary step slices them
+            x, h = self._add_norm(ops.linear(attn.reshape(b, ids.shape[1], -1), lw["o_proj"], defer=not boundary),
+                                  x, lw["post_attention_layernorm"])
+            delta = self._mlp(lw, h, defer=not boundary)
         cache.reset_chunk_counter()
+        if not boundary:
+            return self._logits(x, delta)
         return self._logits(x[:, :1], delta[:, :1])
 
     # ---- decode through a HIP graph ----------------------------------------------------
@@ -367,8 +372,9 @@ class KsaQwen3ForCausalLM:
                                         kv_out_row=st["cur"][kind, 0])
             attn = ops.decode(q.transpose(1, 2), cache.key_cache[li], cache.value_cache[li],
                               st["cur"][kind, 1], st["cur"][kind, 2], self.scaling)
-            x, h = self._add_norm(ops.linear(attn.reshape(b, 1, -1), lw["o_proj"]), x, lw["post_attention_layernorm"])
-            delta = self._mlp(lw, h)
+            x, h = self._add_norm(ops.linear(attn.reshape(b, 1, -1), lw["o_proj"], defer=True), x,
+                                  lw["post_attention_layernorm"])
+            delta = self._mlp(lw, h, defer=True)
         return self._logits(x, delta)
 
     @torch.no_grad()

@@ -40,3 +40,33 @@ def test_gpu_linear_rows_views_and_errors():
     with pytest.raises(KsaError):
         linear_rows(torch.zeros(2, 48, dtype=torch.bfloat16, device="cuda"),
                     torch.zeros(8, 48, dtype=torch.bfloat16, device="cuda"))   # K not a multiple of 32
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,N,K", [(8, 2560, 4096), (8, 2560, 9728), (1, 2560, 4096), (16, 1024, 1024), (3, 64, 512),
+                                   (2, 8192, 1024)])
+def test_gpu_deferred_product_into_add_rmsnorm(dtype, M, N, K):
+    """A product left as K-split partial sums and added inside `add_rmsnorm`: the sum with the
+    residual is bit for bit what the reduced product followed by `add_rmsnorm` gives (same
+    summation order over the splits, same rounding points); the normalised output may differ by
+    one unit in the last place in a few elements, because the mean square is summed over a
+    workgroup instead of a wave.  A product that is not split comes back as a plain tensor."""
+    from ksa_amd import add_rmsnorm
+    from ksa_amd.gemm import SplitKPartials, linear_rows
+    g = torch.Generator().manual_seed(M + N + K)
+    x = torch.randn(1, M, K, generator=g).to(dtype).cuda()
+    w = (torch.randn(N, K, generator=g) * 0.05).to(dtype).cuda()
+    res = torch.randn(1, M, N, generator=g).to(dtype).cuda()
+    nw = (1 + 0.1 * torch.randn(N, generator=g)).to(dtype).cuda()
+    s0, h0 = add_rmsnorm(linear_rows(x, w), res, nw, 1e-6)
+    d = linear_rows(x, w, defer=True)
+    if N * K >= 2560 * 4096:
+        assert isinstance(d, SplitKPartials) and d.shape == (1, M, N)
+    s1, h1 = add_rmsnorm(d, res, nw, 1e-6)
+    assert s1.shape == s0.shape and torch.equal(s0, s1)
+    a, b = h0.float().flatten(), h1.float().flatten()
+    mant = 7 if dtype == torch.bfloat16 else 10
+    ulp = torch.exp2(torch.floor(torch.log2(a.abs().clamp_min(2.0 ** -14))) - mant)
+    assert ((a - b).abs() <= ulp * 1.01).all()
+    assert (a != b).float().mean() <= 0.01
