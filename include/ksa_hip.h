@@ -157,6 +157,13 @@ int ksa_silu_mul(const void* gate, const void* up, void* out, long long rows, in
                  long long gate_row_stride, long long up_row_stride, long long out_row_stride,
                  int dtype, void* stream);
 
+/* ksa_silu_mul whose gate | up is still the K-split partial sums of the fused gate_up projection
+ * (fp32 [ksplit][16][2 I], left by ksa_gemm_rows called with out == NULL): both halves are summed
+ * in split order and rounded first, so the result is bit-identical to the two-kernel form.
+ * rows <= 16. */
+int ksa_silu_mul_partials(const float* partials, int ksplit, void* out, int rows, int I,
+                          long long out_row_stride, int dtype, void* stream);
+
 /* y = x W^T for at most 16 rows of x (decode steps), bound by the weight bytes.
  * Replaces torch.nn.functional.linear at the projections of a decode step (HF:628-641 q/k/v and
  * o projections, HF:507-514 MLP, HF:1338 lm_head), bias-free as in the reference's config.
@@ -165,7 +172,7 @@ int ksa_silu_mul(const void* gate, const void* up, void* out, long long rows, in
  * ksplit > 1 splits K over workgroups (ksa_gemm_rows_auto_splits) and needs
  * ksa_gemm_rows_workspace_bytes(N, ksplit) bytes of device workspace.  With ksplit > 1 out may
  * be NULL: the partial sums (fp32 [ksplit][16][N]) are then left in the workspace for a consumer
- * that adds them itself (ksa_add_rmsnorm_partials). */
+ * that adds them itself (ksa_add_rmsnorm_partials, ksa_silu_mul_partials). */
 int ksa_gemm_rows_auto_splits(int N, int K);
 size_t ksa_gemm_rows_workspace_bytes(int N, int ksplit);
 int ksa_gemm_rows(const void* x, const void* w, void* out, int M, int N, int K, long long x_row_stride,

@@ -190,17 +190,54 @@ struct ActParams {
     uint16_t* out;
     int64_t gs, us, os;  // row strides (elements)
     int I;
+    const float* part;   // if set: gate | up as K-split partial sums, see the kernel
+    int ksplit;
 };
 
 // blockIdx.x = row, blockIdx.y = block of 256 16-byte items inside the row
+// eight consecutive columns of a row of x = the rounded sum of fp32 slices [ksplit][16][width]
+// (the K-split partial sums of ksa_gemm_rows), added in split order like its own reduction
+template <typename T>
+__device__ __forceinline__ u32x4 ksa_sum_partials8(const float* part, int ksplit, int width, int row, int col) {
+    using C = KsaCvt<T>;
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int sp0 = 0; sp0 < ksplit; sp0 += 8) {  // eight slices requested together
+        f32x4 lo[8], hi[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int sp = min(sp0 + u, ksplit - 1);
+            const float* src = part + ((int64_t)sp * 16 + row) * width + col;
+            lo[u] = *reinterpret_cast<const f32x4*>(src);
+            hi[u] = *reinterpret_cast<const f32x4*>(src + 4);
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            if (sp0 + u < ksplit) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[i] += lo[u][i], acc[4 + i] += hi[u][i];
+            }
+        }
+    }
+    u32x4 r;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r[i] = C::down2(acc[2 * i], acc[2 * i + 1]);
+    return r;
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void ksa_silu_mul_kernel(const ActParams p) {
     using C = KsaCvt<T>;
     const int64_t row = blockIdx.x;
     const int idx = blockIdx.y * 256 + threadIdx.x;
     if (idx >= p.I / 8) return;
-    const u32x4 g = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.gate + row * p.gs + 8 * idx));
-    const u32x4 u = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.up + row * p.us + 8 * idx));
+    u32x4 g, u;
+    if (p.part) {  // gate | up still as the partial sums of the fused projection [ksplit][16][2 I]
+        g = ksa_sum_partials8<T>(p.part, p.ksplit, 2 * p.I, (int)row, 8 * idx);
+        u = ksa_sum_partials8<T>(p.part, p.ksplit, 2 * p.I, (int)row, p.I + 8 * idx);
+    } else {
+        g = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.gate + row * p.gs + 8 * idx));
+        u = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.up + row * p.us + 8 * idx));
+    }
     u32x4 o;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -277,7 +314,25 @@ extern "C" int ksa_silu_mul(const void* gate, const void* up, void* out, long lo
     const int yblocks = (I / 8 + 255) / 256;
     if (yblocks > 65535) return KSA_ERR_INVALID;
     ActParams p{(const uint16_t*)gate, (const uint16_t*)up, (uint16_t*)out, gate_row_stride, up_row_stride,
-                out_row_stride, I};
+                out_row_stride, I, nullptr, 0};
+    if (dtype == KSA_DTYPE_BF16)
+        hipLaunchKernelGGL(ksa_silu_mul_kernel<KsaBf16>, dim3((unsigned)rows, yblocks), dim3(256), 0,
+                           (hipStream_t)stream, p);
+    else
+        hipLaunchKernelGGL(ksa_silu_mul_kernel<KsaF16>, dim3((unsigned)rows, yblocks), dim3(256), 0,
+                           (hipStream_t)stream, p);
+    return ksa_check_launch();
+}
+
+extern "C" int ksa_silu_mul_partials(const float* partials, int ksplit, void* out, int rows, int I,
+                                     long long out_row_stride, int dtype, void* stream) {
+    if (!partials || !out) return KSA_ERR_NULL;
+    if (rows <= 0 || rows > 16 || ksplit < 1 || ksplit > 64 || I <= 0 || I % 8 != 0) return KSA_ERR_INVALID;
+    if (dtype != KSA_DTYPE_BF16 && dtype != KSA_DTYPE_F16) return KSA_ERR_UNSUPPORTED;
+    if (!al16(partials) || !al16(out) || out_row_stride % 8) return KSA_ERR_ALIGN;
+    const int yblocks = (I / 8 + 255) / 256;
+    if (yblocks > 65535) return KSA_ERR_INVALID;
+    ActParams p{nullptr, nullptr, (uint16_t*)out, 0, 0, out_row_stride, I, partials, ksplit};
     if (dtype == KSA_DTYPE_BF16)
         hipLaunchKernelGGL(ksa_silu_mul_kernel<KsaBf16>, dim3((unsigned)rows, yblocks), dim3(256), 0,
                            (hipStream_t)stream, p);

@@ -75,8 +75,23 @@ def add_rmsnorm(x: torch.Tensor, residual: Optional[torch.Tensor], weight: torch
     return s.view(x.shape), out.view(x.shape)
 
 
-def silu_mul(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
-    """round(silu(gate)) * up; gate and up may be strided views (halves of one GEMM output)."""
+def silu_mul(gate, up: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """round(silu(gate)) * up; gate and up may be strided views (halves of one GEMM output).
+    With `up` left out, `gate` is the whole gate | up projection [..., 2 I]: a tensor, or the
+    `SplitKPartials` of a deferred `linear_rows`, whose partial sums are then added here."""
+    if isinstance(gate, SplitKPartials):
+        assert up is None
+        x = gate
+        I = x.shape[-1] // 2
+        out = torch.empty(x.rows, I, dtype=x.dtype, device=x.device)
+        with torch.cuda.device(x.device):
+            rc = _lib.lib().ksa_silu_mul_partials(x.workspace.data_ptr(), x.ksplit, out.data_ptr(), x.rows, I,
+                                                  out.stride(0), _DT[x.dtype], _lib.stream_ptr(x.device))
+        _lib.check(rc, "ksa_silu_mul_partials")
+        return out.view(*x.shape[:-1], I)
+    if up is None:
+        I = gate.shape[-1] // 2
+        gate, up = gate[..., :I], gate[..., I:]
     assert gate.is_cuda and gate.dtype in _DT and up.dtype == gate.dtype and gate.shape == up.shape
     I = gate.shape[-1]
     g2, u2 = _rows2d(gate), _rows2d(up)

@@ -261,9 +261,8 @@ class KsaQwen3ForCausalLM:
 
     def _mlp(self, lw, x, defer=False):
         """`defer`: the result only goes to `_add_norm` (see `HipOps.linear`)."""
-        gu = self.ops.linear(x, lw["gate_up_proj"])
-        I = self.config.intermediate_size
-        return self.ops.linear(self.ops.silu_mul(gu[..., :I], gu[..., I:]), lw["down_proj"], defer=defer)
+        gu = self.ops.linear(x, lw["gate_up_proj"], defer=defer)
+        return self.ops.linear(self.ops.silu_mul(gu), lw["down_proj"], defer=defer)
 
     def _logits(self, x_last, delta_last):
         _, h = self._add_norm(delta_last, x_last, self.w["norm"])

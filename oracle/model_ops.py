@@ -49,7 +49,12 @@ class OracleOps:
     def linear(x, weight, defer=False):  # `defer` is a launch-count hint of the GPU operators
         return torch.nn.functional.linear(x, weight)
     add_rmsnorm = staticmethod(cpu_path.add_rmsnorm)
-    silu_mul = staticmethod(cpu_path.silu_mul)
+    @staticmethod
+    def silu_mul(gate, up=None):
+        if up is None:  # the whole gate | up projection
+            I = gate.shape[-1] // 2
+            gate, up = gate[..., :I], gate[..., I:]
+        return cpu_path.silu_mul(gate, up)
 
     @staticmethod
     def summary_attn_func(q, k, v, C, S, W, summary_pos=None):

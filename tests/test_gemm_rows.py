@@ -70,3 +70,24 @@ def test_gpu_deferred_product_into_add_rmsnorm(dtype, M, N, K):
     ulp = torch.exp2(torch.floor(torch.log2(a.abs().clamp_min(2.0 ** -14))) - mant)
     assert ((a - b).abs() <= ulp * 1.01).all()
     assert (a != b).float().mean() <= 0.01
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,I,K", [(8, 9728, 2560), (1, 9728, 2560), (16, 520, 1024), (5, 64, 512)])
+def test_gpu_deferred_gate_up_into_silu_mul(dtype, M, I, K):
+    """gate | up left as K-split partial sums and added inside `silu_mul`: bit for bit the
+    two-kernel result (the halves are summed in split order and rounded before the activation)."""
+    from ksa_amd import silu_mul
+    from ksa_amd.gemm import SplitKPartials, linear_rows
+    g = torch.Generator().manual_seed(M + I + K)
+    x = torch.randn(1, M, K, generator=g).to(dtype).cuda()
+    w = (torch.randn(2 * I, K, generator=g) * 0.05).to(dtype).cuda()
+    gu = linear_rows(x, w)
+    want = silu_mul(gu[..., :I], gu[..., I:])
+    assert torch.equal(silu_mul(gu), want)                     # whole projection as one tensor
+    d = linear_rows(x, w, defer=True)
+    if I >= 9728:
+        assert isinstance(d, SplitKPartials)
+    got = silu_mul(d)
+    assert got.shape == want.shape and torch.equal(got, want)
