@@ -126,6 +126,17 @@ int ksa_pre_attention(const void* q, const void* k, const void* v, const void* q
                       const int64_t* v_out_strides, const int64_t* cos_strides,
                       const int32_t* kv_out_row_seq, float eps, void* stream);
 
+/* ksa_pre_attention whose q | k | v rows are still the K-split partial sums of the fused qkv
+ * projection (fp32 [ksplit][16][(Hq + 2 Hkv) D], left by ksa_gemm_rows called with out == NULL;
+ * row = batch index * S + position): summed in split order and rounded first, so the outputs are
+ * bit-identical to the two-kernel form.  batch * S <= 16. */
+int ksa_pre_attention_partials(const float* partials, int ksplit, const void* q_weight,
+                               const void* k_weight, const void* cos, const void* sin, void* q_out,
+                               void* k_out, void* v_out, int batch, int S, int Hq, int Hkv, int D,
+                               int dtype, const int64_t* q_out_strides, const int64_t* k_out_strides,
+                               const int64_t* v_out_strides, const int64_t* cos_strides,
+                               const int32_t* kv_out_row_seq, float eps, void* stream);
+
 /* Residual add + RMSNorm over the hidden size, one pass.
  * Replaces Qwen3RMSNorm.forward (HF:64-79: fp32 normalisation, rounded to the 16-bit type, times
  * the 16-bit weight) together with the residual add in front of it (HF:946, :952).
@@ -172,7 +183,8 @@ int ksa_silu_mul_partials(const float* partials, int ksplit, void* out, int rows
  * ksplit > 1 splits K over workgroups (ksa_gemm_rows_auto_splits) and needs
  * ksa_gemm_rows_workspace_bytes(N, ksplit) bytes of device workspace.  With ksplit > 1 out may
  * be NULL: the partial sums (fp32 [ksplit][16][N]) are then left in the workspace for a consumer
- * that adds them itself (ksa_add_rmsnorm_partials, ksa_silu_mul_partials). */
+ * that adds them itself (ksa_add_rmsnorm_partials, ksa_silu_mul_partials,
+ * ksa_pre_attention_partials). */
 int ksa_gemm_rows_auto_splits(int N, int K);
 size_t ksa_gemm_rows_workspace_bytes(int N, int ksplit);
 int ksa_gemm_rows(const void* x, const void* w, void* out, int M, int N, int K, long long x_row_stride,

@@ -81,3 +81,33 @@ struct KsaCvt<KsaF16> {
     static constexpr uint32_t kOnes = 0x3c003c00u;
 };
 
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// eight consecutive columns of a row of x = the rounded sum of fp32 slices [ksplit][16][width]
+// (the K-split partial sums of ksa_gemm_rows), added in split order like its own reduction
+template <typename T>
+__device__ __forceinline__ u32x4 ksa_sum_partials8(const float* part, int ksplit, int width, int row, int col) {
+    using C = KsaCvt<T>;
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int sp0 = 0; sp0 < ksplit; sp0 += 8) {  // eight slices requested together
+        f32x4 lo[8], hi[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int sp = min(sp0 + u, ksplit - 1);
+            const float* src = part + ((int64_t)sp * 16 + row) * width + col;
+            lo[u] = *reinterpret_cast<const f32x4*>(src);
+            hi[u] = *reinterpret_cast<const f32x4*>(src + 4);
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            if (sp0 + u < ksplit) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[i] += lo[u][i], acc[4 + i] += hi[u][i];
+            }
+        }
+    }
+    u32x4 r;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r[i] = C::down2(acc[2 * i], acc[2 * i + 1]);
+    return r;
+}

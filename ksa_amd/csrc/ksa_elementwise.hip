@@ -14,8 +14,6 @@
 
 namespace {
 
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-
 struct NormParams {
     const uint16_t* x;
     const float* part;     // partial-sum variant: x = rounded sum of `ksplit` fp32 slices [ksplit][16][H]
@@ -195,43 +193,15 @@ struct ActParams {
 };
 
 // blockIdx.x = row, blockIdx.y = block of 256 16-byte items inside the row
-// eight consecutive columns of a row of x = the rounded sum of fp32 slices [ksplit][16][width]
-// (the K-split partial sums of ksa_gemm_rows), added in split order like its own reduction
-template <typename T>
-__device__ __forceinline__ u32x4 ksa_sum_partials8(const float* part, int ksplit, int width, int row, int col) {
-    using C = KsaCvt<T>;
-    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    for (int sp0 = 0; sp0 < ksplit; sp0 += 8) {  // eight slices requested together
-        f32x4 lo[8], hi[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            const int sp = min(sp0 + u, ksplit - 1);
-            const float* src = part + ((int64_t)sp * 16 + row) * width + col;
-            lo[u] = *reinterpret_cast<const f32x4*>(src);
-            hi[u] = *reinterpret_cast<const f32x4*>(src + 4);
-        }
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            if (sp0 + u < ksplit) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i) acc[i] += lo[u][i], acc[4 + i] += hi[u][i];
-            }
-        }
-    }
-    u32x4 r;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) r[i] = C::down2(acc[2 * i], acc[2 * i + 1]);
-    return r;
-}
-
-template <typename T>
+// kPartials: a variant of its own, so that the streaming variant does not carry its registers
+template <typename T, bool kPartials>
 __global__ __launch_bounds__(256) void ksa_silu_mul_kernel(const ActParams p) {
     using C = KsaCvt<T>;
     const int64_t row = blockIdx.x;
     const int idx = blockIdx.y * 256 + threadIdx.x;
     if (idx >= p.I / 8) return;
     u32x4 g, u;
-    if (p.part) {  // gate | up still as the partial sums of the fused projection [ksplit][16][2 I]
+    if constexpr (kPartials) {  // gate | up still as the partial sums of the fused projection [ksplit][16][2 I]
         g = ksa_sum_partials8<T>(p.part, p.ksplit, 2 * p.I, (int)row, 8 * idx);
         u = ksa_sum_partials8<T>(p.part, p.ksplit, 2 * p.I, (int)row, p.I + 8 * idx);
     } else {
@@ -316,10 +286,10 @@ extern "C" int ksa_silu_mul(const void* gate, const void* up, void* out, long lo
     ActParams p{(const uint16_t*)gate, (const uint16_t*)up, (uint16_t*)out, gate_row_stride, up_row_stride,
                 out_row_stride, I, nullptr, 0};
     if (dtype == KSA_DTYPE_BF16)
-        hipLaunchKernelGGL(ksa_silu_mul_kernel<KsaBf16>, dim3((unsigned)rows, yblocks), dim3(256), 0,
+        hipLaunchKernelGGL((ksa_silu_mul_kernel<KsaBf16, false>), dim3((unsigned)rows, yblocks), dim3(256), 0,
                            (hipStream_t)stream, p);
     else
-        hipLaunchKernelGGL(ksa_silu_mul_kernel<KsaF16>, dim3((unsigned)rows, yblocks), dim3(256), 0,
+        hipLaunchKernelGGL((ksa_silu_mul_kernel<KsaF16, false>), dim3((unsigned)rows, yblocks), dim3(256), 0,
                            (hipStream_t)stream, p);
     return ksa_check_launch();
 }
@@ -334,10 +304,10 @@ extern "C" int ksa_silu_mul_partials(const float* partials, int ksplit, void* ou
     if (yblocks > 65535) return KSA_ERR_INVALID;
     ActParams p{nullptr, nullptr, (uint16_t*)out, 0, 0, out_row_stride, I, partials, ksplit};
     if (dtype == KSA_DTYPE_BF16)
-        hipLaunchKernelGGL(ksa_silu_mul_kernel<KsaBf16>, dim3((unsigned)rows, yblocks), dim3(256), 0,
+        hipLaunchKernelGGL((ksa_silu_mul_kernel<KsaBf16, true>), dim3((unsigned)rows, yblocks), dim3(256), 0,
                            (hipStream_t)stream, p);
     else
-        hipLaunchKernelGGL(ksa_silu_mul_kernel<KsaF16>, dim3((unsigned)rows, yblocks), dim3(256), 0,
+        hipLaunchKernelGGL((ksa_silu_mul_kernel<KsaF16, true>), dim3((unsigned)rows, yblocks), dim3(256), 0,
                            (hipStream_t)stream, p);
     return ksa_check_launch();
 }

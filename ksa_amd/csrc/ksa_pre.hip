@@ -29,6 +29,8 @@ struct PreParams {
     uint16_t* dst[3];         // q, k, v outputs
     const uint16_t* w[2];     // q_norm, k_norm weights [D]
     const int32_t* kv_row;    // [batch] or null: row added to the k / v destination of a sequence
+    const float* part;        // if set: q | k | v rows as K-split partial sums [ksplit][16][(Hq + 2 Hkv) D], src unused
+    int ksplit;
     const uint16_t* cos;      // [batch or 1, S, D]
     const uint16_t* sin;
     int64_t s_bs[3], s_rs[3], s_hs[3];
@@ -72,7 +74,9 @@ __device__ __forceinline__ float pre_row_sum(float ss) {
 // packed dot products against operands that hold one element and a zero, straight from the
 // packed words (exact in fp32), and the final sum of the two rounded terms is a dot product
 // with (1, 1).
-template <typename T, int D>
+// kPartials: the rows come as K-split partial sums (a variant of its own, so that the streaming
+// variant does not carry its registers).
+template <typename T, int D, bool kPartials>
 __global__ __launch_bounds__(256) void ksa_pre_attention_kernel(const PreParams p) {
     using C = PreCvt<T>;
     constexpr int LPR = D / 8;          // lanes per head row
@@ -123,6 +127,7 @@ __global__ __launch_bounds__(256) void ksa_pre_attention_kernel(const PreParams 
     struct Group {
         bool live;             // wave-uniform: there is such a group
         int which, tok, h0;
+        int col0;              // partial-sum input: first column of the group's first head
         const uint16_t* sbase;
         uint16_t* dbase;
     };
@@ -146,6 +151,7 @@ __global__ __launch_bounds__(256) void ksa_pre_attention_kernel(const PreParams 
         }
         g.which = gi < Gq ? 0 : (gi < Gq + Gk ? 1 : 2);
         g.h0 = (gi - (g.which == 0 ? 0 : (g.which == 1 ? Gq : Gq + Gk))) * RPW;
+        g.col0 = ((g.which == 0 ? 0 : (g.which == 1 ? p.Hq : p.Hq + p.Hkv)) + g.h0) * D;
         g.sbase = p.src[g.which] + nb * p.s_bs[g.which] + (int64_t)ns * p.s_rs[g.which] + (int64_t)g.h0 * p.s_hs[g.which];
         // (k and v may go to a row of their sequence that the host does not know: a cache cursor)
         const int64_t drow = ns + ((g.which != 0 && p.kv_row) ? p.kv_row[nb] : 0);
@@ -157,6 +163,13 @@ __global__ __launch_bounds__(256) void ksa_pre_attention_kernel(const PreParams 
     // a lane group beyond the last head is idle as a whole, exchange partners included
     auto lane_ok = [&](const Group& g) { return g.h0 + sub < (g.which == 0 ? p.Hq : p.Hkv); };
     const u32x4 zero4 = {0u, 0u, 0u, 0u};
+    // this lane's 16 bytes of a group's rows: from the projection output, or (decode steps) from
+    // the K-split partial sums of the projection, added and rounded as its own reduction would
+    auto fetch = [&](const Group& g) {
+        if constexpr (kPartials)
+            return ksa_sum_partials8<T>(p.part, p.ksplit, (p.Hq + 2 * p.Hkv) * D, g.tok, g.col0 + sub * D + 8 * t);
+        return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(g.sbase + pick(g.which, lsrc)));
+    };
 
     Group g = next_group();
     u32x4 raw = zero4, craw = zero4, sraw = zero4;
@@ -164,7 +177,7 @@ __global__ __launch_bounds__(256) void ksa_pre_attention_kernel(const PreParams 
         craw = *reinterpret_cast<const u32x4*>(p.cos + nb * p.c_bs + (int64_t)ns * p.c_rs + 8 * t);
         sraw = *reinterpret_cast<const u32x4*>(p.sin + nb * p.c_bs + (int64_t)ns * p.c_rs + 8 * t);
         // every byte of q, k, v is touched once: non-temporal accesses
-        if (lane_ok(g)) raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(g.sbase + pick(g.which, lsrc)));
+        if (lane_ok(g)) raw = fetch(g);
     }
     int cur = -1;  // token whose rotary row is split below
     uint32_t clo[4], chi[4], slo[4], shi[4];
@@ -176,7 +189,7 @@ __global__ __launch_bounds__(256) void ksa_pre_attention_kernel(const PreParams 
                 craw_n = *reinterpret_cast<const u32x4*>(p.cos + nb * p.c_bs + (int64_t)ns * p.c_rs + 8 * t);
                 sraw_n = *reinterpret_cast<const u32x4*>(p.sin + nb * p.c_bs + (int64_t)ns * p.c_rs + 8 * t);
             }
-            if (lane_ok(n)) raw_n = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(n.sbase + pick(n.which, lsrc)));
+            if (lane_ok(n)) raw_n = fetch(n);
         }
         if (g.tok != cur) {  // wave-uniform: the rotary row of this token, split like the weights
             cur = g.tok;
@@ -242,11 +255,24 @@ int launch_pre(PreParams p, hipStream_t stream) {
     // addresses in flight narrow: measured 5 % faster than a grid-stride loop of long-lived
     // workgroups over the same accesses (a plain copy shows the same preference, 6.2 against
     // 4.9 TB/s).  Four passes amortise a workgroup's set-up; 2 .. 8 measure alike.
-    p.passes_per_wg = 4;
+    // (a handful of tokens - a decode step - get one pass per workgroup: all the parallelism there is)
+    p.passes_per_wg = (int64_t)p.batch * p.S / p.tok_per_pass >= 4 * 1024 ? 4 : 1;
     const int64_t span = (int64_t)p.passes_per_wg * p.tok_per_pass;
     const int64_t blocks = ((int64_t)p.batch * p.S + span - 1) / span;
-    hipLaunchKernelGGL((ksa_pre_attention_kernel<T, D>), dim3((unsigned)blocks), dim3(256), 0, stream, p);
+    if (p.part)
+        hipLaunchKernelGGL((ksa_pre_attention_kernel<T, D, true>), dim3((unsigned)blocks), dim3(256), 0, stream, p);
+    else
+        hipLaunchKernelGGL((ksa_pre_attention_kernel<T, D, false>), dim3((unsigned)blocks), dim3(256), 0, stream, p);
     return ksa_check_launch();
+}
+
+int dispatch_pre(const PreParams& p, int D, int dtype, hipStream_t stp) {
+    if (dtype == KSA_DTYPE_BF16) {
+        if (D == 128) return launch_pre<KsaBf16, 128>(p, stp);
+        return launch_pre<KsaBf16, 64>(p, stp);
+    }
+    if (D == 128) return launch_pre<KsaF16, 128>(p, stp);
+    return launch_pre<KsaF16, 64>(p, stp);
 }
 
 }  // namespace
@@ -295,11 +321,45 @@ extern "C" int ksa_pre_attention(const void* q, const void* k, const void* v, co
     p.c_bs = cos_strides[0], p.c_rs = cos_strides[1];
     p.batch = batch, p.S = S, p.Hq = Hq, p.Hkv = Hkv;
     p.eps = eps;
-    hipStream_t stp = (hipStream_t)stream;
-    if (dtype == KSA_DTYPE_BF16) {
-        if (D == 128) return launch_pre<KsaBf16, 128>(p, stp);
-        return launch_pre<KsaBf16, 64>(p, stp);
+    return dispatch_pre(p, D, dtype, (hipStream_t)stream);
+}
+
+extern "C" int ksa_pre_attention_partials(const float* partials, int ksplit, const void* q_weight,
+                                          const void* k_weight, const void* cos, const void* sin, void* q_out,
+                                          void* k_out, void* v_out, int batch, int S, int Hq, int Hkv, int D,
+                                          int dtype, const int64_t* q_out_strides, const int64_t* k_out_strides,
+                                          const int64_t* v_out_strides, const int64_t* cos_strides,
+                                          const int32_t* kv_out_row_seq, float eps, void* stream) {
+    if (!partials || !q_weight || !k_weight || !cos || !sin || !q_out || !k_out || !v_out) return KSA_ERR_NULL;
+    if (!q_out_strides || !k_out_strides || !v_out_strides || !cos_strides) return KSA_ERR_NULL;
+    if (batch <= 0 || S <= 0 || (int64_t)batch * S > 16 || Hq <= 0 || Hkv <= 0 || ksplit < 1 || ksplit > 64 ||
+        !(eps >= 0.f))
+        return KSA_ERR_INVALID;
+    for (const int64_t* s3 : {q_out_strides, k_out_strides, v_out_strides})
+        if (s3[2] < 0 || s3[2] * 8 + 128 >= (1ll << 32)) return KSA_ERR_INVALID;
+    if (dtype != KSA_DTYPE_BF16 && dtype != KSA_DTYPE_F16) return KSA_ERR_UNSUPPORTED;
+    if (D != 64 && D != 128) return KSA_ERR_UNSUPPORTED;
+    const void* ptrs[] = {partials, q_weight, k_weight, cos, sin, q_out, k_out, v_out};
+    for (const void* ptr : ptrs)
+        if (reinterpret_cast<uintptr_t>(ptr) & 15) return KSA_ERR_ALIGN;
+    for (const int64_t* s3 : {q_out_strides, k_out_strides, v_out_strides})
+        for (int i = 0; i < 3; ++i)
+            if (s3[i] % 8) return KSA_ERR_ALIGN;
+    if (cos_strides[0] % 8 || cos_strides[1] % 8) return KSA_ERR_ALIGN;
+    PreParams p{};
+    p.part = partials;
+    p.ksplit = ksplit;
+    p.dst[0] = (uint16_t*)q_out, p.dst[1] = (uint16_t*)k_out, p.dst[2] = (uint16_t*)v_out;
+    p.w[0] = (const uint16_t*)q_weight, p.w[1] = (const uint16_t*)k_weight;
+    p.cos = (const uint16_t*)cos, p.sin = (const uint16_t*)sin;
+    p.kv_row = kv_out_row_seq;
+    const int64_t* out[] = {q_out_strides, k_out_strides, v_out_strides};
+    for (int i = 0; i < 3; ++i) {
+        p.s_hs[i] = D;  // (only the lane offsets are derived from it; the source is `partials`)
+        p.d_bs[i] = out[i][0], p.d_rs[i] = out[i][1], p.d_hs[i] = out[i][2];
     }
-    if (D == 128) return launch_pre<KsaF16, 128>(p, stp);
-    return launch_pre<KsaF16, 64>(p, stp);
+    p.c_bs = cos_strides[0], p.c_rs = cos_strides[1];
+    p.batch = batch, p.S = S, p.Hq = Hq, p.Hkv = Hkv;
+    p.eps = eps;
+    return dispatch_pre(p, D, dtype, (hipStream_t)stream);
 }

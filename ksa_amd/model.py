@@ -132,6 +132,7 @@ class HipOps:
         from . import cache, decode, elementwise, gemm, pre, prefill
         self.cache_cls = cache.Qwen3RingBufferCache
         self.pre_attention = pre.pre_attention
+        self.pre_attention_partials = pre.pre_attention_partials
         self.summary_attn_func = prefill.summary_attn_func
         self.add_rmsnorm = elementwise.add_rmsnorm
         self.silu_mul = elementwise.silu_mul
@@ -253,6 +254,11 @@ class KsaQwen3ForCausalLM:
         if (cfg.summary_independent_parameters and cfg.mix_coeff != 0 and summary_rows is not None
                 and summary_rows.numel() > 0):
             qkv[:, summary_rows] = self.ops.linear(h[:, summary_rows], lw["qkv_proj_summary"])
+        return self._split_qkv(qkv)
+
+    def _split_qkv(self, qkv):
+        cfg = self.config
+        D, Hq, Hkv = cfg.head_dim, cfg.num_attention_heads, cfg.num_key_value_heads
         b, L, _ = qkv.shape
         q = qkv[..., : Hq * D].view(b, L, Hq, D)
         k = qkv[..., Hq * D: (Hq + Hkv) * D].view(b, L, Hkv, D)
@@ -363,12 +369,17 @@ class KsaQwen3ForCausalLM:
         for li, lw in enumerate(self.w["layers"]):
             kind = 1 if cache.is_large_window[li] else 0
             x, h = self._add_norm(delta, x, lw["input_layernorm"])
-            q, k, v = self._qkv(lw, h, None)
             # k and v go straight to the cache row the device-side cursor names
-            q, _, _ = ops.pre_attention(q, k, v, lw["q_norm"], lw["k_norm"], cos, sin, cfg.rms_norm_eps,
-                                        k_out=cache.key_cache[li][:, :, :1].transpose(1, 2),
-                                        v_out=cache.value_cache[li][:, :, :1].transpose(1, 2),
-                                        kv_out_row=st["cur"][kind, 0])
+            slots = dict(k_out=cache.key_cache[li][:, :, :1].transpose(1, 2),
+                         v_out=cache.value_cache[li][:, :, :1].transpose(1, 2), kv_out_row=st["cur"][kind, 0])
+            qkv = ops.linear(h, lw["qkv_proj"], defer=True)
+            if torch.is_tensor(qkv):
+                q, k, v = self._split_qkv(qkv)
+                q, _, _ = ops.pre_attention(q, k, v, lw["q_norm"], lw["k_norm"], cos, sin, cfg.rms_norm_eps, **slots)
+            else:  # still the K-split partial sums of the projection: added inside the kernel
+                q, _, _ = ops.pre_attention_partials(qkv, cfg.num_attention_heads, cfg.num_key_value_heads,
+                                                     cfg.head_dim, lw["q_norm"], lw["k_norm"], cos, sin,
+                                                     cfg.rms_norm_eps, **slots)
             attn = ops.decode(q.transpose(1, 2), cache.key_cache[li], cache.value_cache[li],
                               st["cur"][kind, 1], st["cur"][kind, 2], self.scaling)
             x, h = self._add_norm(ops.linear(attn.reshape(b, 1, -1), lw["o_proj"], defer=True), x,

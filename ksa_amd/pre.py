@@ -72,3 +72,46 @@ def pre_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q_norm_weig
                                  float(eps), _lib.stream_ptr(q.device))
     _lib.check(rc, "ksa_pre_attention")
     return qo, ko, vo
+
+
+def pre_attention_partials(qkv, Hq: int, Hkv: int, D: int, q_norm_weight: torch.Tensor,
+                           k_norm_weight: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, eps: float = 1e-6,
+                           q_out: Optional[torch.Tensor] = None, k_out: Optional[torch.Tensor] = None,
+                           v_out: Optional[torch.Tensor] = None,
+                           kv_out_row: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """`pre_attention` on a fused q | k | v projection [b, S, (Hq + 2 Hkv) D] that is still the
+    `SplitKPartials` of a deferred `linear_rows` (at most 16 rows): the partial sums are added
+    inside the kernel, with the outputs of the two-kernel form."""
+    from .gemm import SplitKPartials
+    assert isinstance(qkv, SplitKPartials) and len(qkv.shape) == 3 and qkv.shape[-1] == (Hq + 2 * Hkv) * D
+    b, S = qkv.shape[0], qkv.shape[1]
+    dev, dtype = qkv.device, qkv.dtype
+    if cos.dim() == 2:
+        cos, sin = cos[None], sin[None]
+    assert cos.shape[-2:] == (S, D) and sin.shape == cos.shape and cos.shape[0] in (1, b)
+    cos = cos.to(dtype).contiguous()
+    sin = sin.to(dtype).contiguous()
+    qw = q_norm_weight.to(dtype).contiguous()
+    kw = k_norm_weight.to(dtype).contiguous()
+    assert qw.shape == (D,) and kw.shape == (D,)
+    outs = []
+    for given, H in ((q_out, Hq), (k_out, Hkv), (v_out, Hkv)):
+        if given is None:
+            given = torch.empty(b, S, H, D, dtype=dtype, device=dev)
+        assert given.shape == (b, S, H, D) and given.dtype == dtype and given.stride(3) == 1
+        outs.append(given)
+    qo, ko, vo = outs
+    if kv_out_row is not None:
+        assert kv_out_row.is_cuda and kv_out_row.dtype == torch.int32 and kv_out_row.shape == (b,) \
+            and kv_out_row.is_contiguous(), "kv_out_row must be a contiguous int32 [b] GPU tensor"
+        assert k_out is not None and v_out is not None, "kv_out_row needs k_out and v_out"
+    cstr = (ctypes.c_int64 * 3)(cos.stride(0) if cos.shape[0] > 1 else 0, cos.stride(1), 0)
+    L = _lib.lib()
+    with torch.cuda.device(dev):
+        rc = L.ksa_pre_attention_partials(qkv.workspace.data_ptr(), qkv.ksplit, qw.data_ptr(), kw.data_ptr(),
+                                          cos.data_ptr(), sin.data_ptr(), qo.data_ptr(), ko.data_ptr(),
+                                          vo.data_ptr(), b, S, Hq, Hkv, D, _DT[dtype], _bsh(qo), _bsh(ko),
+                                          _bsh(vo), cstr, None if kv_out_row is None else kv_out_row.data_ptr(),
+                                          float(eps), _lib.stream_ptr(dev))
+    _lib.check(rc, "ksa_pre_attention_partials")
+    return qo, ko, vo

@@ -195,3 +195,45 @@ def test_pre_attention_rejects_bad_inputs():
         ksa_amd.pre_attention(q, q, q, w, w, c, c)
     with pytest.raises(AssertionError):
         ksa_amd.pre_attention(q.float(), q.float(), q.float(), w, w, c, c)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("b,S,Hq,Hkv,D", [(8, 1, 32, 8, 128), (1, 1, 32, 8, 128), (2, 3, 6, 2, 64), (16, 1, 4, 4, 128)])
+def test_pre_attention_gpu_from_split_k_partials(dtype, b, S, Hq, Hkv, D):
+    """q | k | v still as the K-split partial sums of the fused projection: the kernel adds them
+    itself and returns bit for bit what the reduced projection followed by `pre_attention` gives,
+    including the write to a cache row named in device memory."""
+    import ksa_amd
+    from ksa_amd.gemm import SplitKPartials, linear_rows
+    from ksa_amd.pre import pre_attention_partials
+    dev = torch.device("cuda")
+    K = 2560
+    g = torch.Generator().manual_seed(b * 100 + S * 10 + Hq)
+    x = torch.randn(b, S, K, generator=g).to(dtype).to(dev)
+    w = (torch.randn((Hq + 2 * Hkv) * D, K, generator=g) * 0.05).to(dtype).to(dev)
+    qw = (1 + 0.1 * torch.randn(D, generator=g)).to(dtype).to(dev)
+    kw = (1 + 0.1 * torch.randn(D, generator=g)).to(dtype).to(dev)
+    cos, sin, _ = _rope_tables(S, D, dtype=dtype)
+    cos, sin = cos.to(dev), sin.to(dev)
+    qkv = linear_rows(x, w)
+    q = qkv[..., : Hq * D].view(b, S, Hq, D)
+    k = qkv[..., Hq * D: (Hq + Hkv) * D].view(b, S, Hkv, D)
+    v = qkv[..., (Hq + Hkv) * D:].view(b, S, Hkv, D)
+    q0, k0, v0 = ksa_amd.pre_attention(q, k, v, qw, kw, cos, sin, eps=1e-6)
+    d = linear_rows(x, w, defer=True)
+    if not isinstance(d, SplitKPartials):
+        pytest.skip("this shape is not split over K")
+    cap = 32
+    kc = torch.zeros(b, Hkv, cap, D, dtype=dtype, device=dev)
+    vc = torch.zeros_like(kc)
+    cursor = (torch.arange(b, device=dev, dtype=torch.int32) * 3) % (cap - S)
+    q1, _, _ = pre_attention_partials(d, Hq, Hkv, D, qw, kw, cos, sin, eps=1e-6,
+                                      k_out=kc[:, :, :S].transpose(1, 2), v_out=vc[:, :, :S].transpose(1, 2),
+                                      kv_out_row=cursor)
+    torch.cuda.synchronize()
+    assert torch.equal(q0, q1)
+    for i in range(b):
+        r = int(cursor[i])
+        assert torch.equal(kc[i, :, r:r + S].transpose(0, 1), k0[i])
+        assert torch.equal(vc[i, :, r:r + S].transpose(0, 1), v0[i])
