@@ -328,15 +328,22 @@ class KsaQwen3ForCausalLM:
         delta = None
         for li, lw in enumerate(self.w["layers"]):
             x, h = self._add_norm(delta, x, lw["input_layernorm"])
-            q, k, v = self._qkv(lw, h, sum_rows)
             if not boundary:
                 k_slot, v_slot = cache.text_slots(li, b, Hkv, D, self.dtype, self.device)
-                q, _, _ = ops.pre_attention(q, k, v, lw["q_norm"], lw["k_norm"], cos, sin, cfg.rms_norm_eps,
-                                            k_out=k_slot, v_out=v_slot)
+                qkv = ops.linear(h, lw["qkv_proj"], defer=True)
+                if torch.is_tensor(qkv):
+                    q, k, v = self._split_qkv(qkv)
+                    q, _, _ = ops.pre_attention(q, k, v, lw["q_norm"], lw["k_norm"], cos, sin, cfg.rms_norm_eps,
+                                                k_out=k_slot, v_out=v_slot)
+                else:  # still the K-split partial sums of the projection: added inside the kernel
+                    q, _, _ = ops.pre_attention_partials(qkv, cfg.num_attention_heads, Hkv, D, lw["q_norm"],
+                                                         lw["k_norm"], cos, sin, cfg.rms_norm_eps,
+                                                         k_out=k_slot, v_out=v_slot)
                 a, e = cache.attention_range(li)
                 attn = ops.decode(q.transpose(1, 2), cache.key_cache[li], cache.value_cache[li], a, e,
                                   self.scaling)
             else:
+                q, k, v = self._qkv(lw, h, sum_rows)
                 q, k, v = ops.pre_attention(q, k, v, lw["q_norm"], lw["k_norm"], cos, sin, cfg.rms_norm_eps)
                 qh, kh, vh = q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2)
                 cache.update_text(kh[:, :, :1], vh[:, :, :1], li)
