@@ -91,8 +91,13 @@ __global__ __launch_bounds__(256) void ksa_add_rmsnorm_partials_kernel(const Nor
     const int tid = threadIdx.x;
     const int row = blockIdx.x;
     const int items = p.H / 8;
-    u32x4 r[NJ];
+    u32x4 r[NJ], wv[NJ];
     float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {  // the weights do not wait for the mean square
+        const int idx = tid + 256 * j;
+        if (idx < items) wv[j] = *reinterpret_cast<const u32x4*>(p.w + 8 * idx);
+    }
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
         const int idx = tid + 256 * j;
@@ -137,12 +142,11 @@ __global__ __launch_bounds__(256) void ksa_add_rmsnorm_partials_kernel(const Nor
     for (int j = 0; j < NJ; ++j) {
         const int idx = tid + 256 * j;
         if (idx < items) {
-            const u32x4 wv = *reinterpret_cast<const u32x4*>(p.w + 8 * idx);
             u32x4 o;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const uint32_t y = C::down2(C::lo(r[j][i]) * inv, C::hi(r[j][i]) * inv);
-                o[i] = C::down2(C::lo(wv[i]) * C::lo(y), C::hi(wv[i]) * C::hi(y));
+                o[i] = C::down2(C::lo(wv[j][i]) * C::lo(y), C::hi(wv[j][i]) * C::hi(y));
             }
             *reinterpret_cast<u32x4*>(p.out_norm + (int64_t)row * p.ns + 8 * idx) = o;
         }
