@@ -255,15 +255,33 @@ __global__ __launch_bounds__(D) void ksa_decode_merge_kernel(const DecodeParams 
     const int bz = blockIdx.z;
     const int d = threadIdx.x;
     const int64_t base = (((int64_t)bz * p.Hkv + kvh) * p.nsplit) * p.ncols_pad + cg;
+    // the loads of eight splits are requested together (two passes: maximum, then weighted sums)
     float mx = -INFINITY;
-    for (int s = 0; s < p.nsplit; ++s) mx = fmaxf(mx, p.ws_ml[(base + (int64_t)s * p.ncols_pad) * 2]);
+    for (int s0 = 0; s0 < p.nsplit; s0 += 8) {
+        float m[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) m[u] = p.ws_ml[(base + (int64_t)min(s0 + u, p.nsplit - 1) * p.ncols_pad) * 2];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) mx = fmaxf(mx, m[u]);
+    }
     float acc = 0.f, l = 0.f;
-    for (int s = 0; s < p.nsplit; ++s) {
-        const int64_t slot = base + (int64_t)s * p.ncols_pad;
-        const float m = p.ws_ml[slot * 2];
-        const float f = (m == -INFINITY) ? 0.f : ksa_exp2(m - mx);
-        acc += p.ws_o[slot * D + d] * f;
-        l += p.ws_ml[slot * 2 + 1] * f;
+    for (int s0 = 0; s0 < p.nsplit; s0 += 8) {
+        float m[8], ls[8], o[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int64_t slot = base + (int64_t)min(s0 + u, p.nsplit - 1) * p.ncols_pad;
+            m[u] = p.ws_ml[slot * 2];
+            ls[u] = p.ws_ml[slot * 2 + 1];
+            o[u] = p.ws_o[slot * D + d];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            if (s0 + u < p.nsplit) {
+                const float f = (m[u] == -INFINITY) ? 0.f : ksa_exp2(m[u] - mx);
+                acc += o[u] * f;
+                l += ls[u] * f;
+            }
+        }
     }
     const int oq = cg / p.g, og = cg % p.g;
     const float val = l > 0.f ? acc / l : 0.f;
