@@ -82,49 +82,34 @@ __global__ __launch_bounds__(256) void ksa_add_rmsnorm_kernel(const NormParams p
 
 // The same step for the few rows of a decode step when x is still the K-split partial sums of
 // the GEMM that produced it (fp32 [ksplit][16][H], as ksa_gemm_rows leaves them): one workgroup
-// per row adds the slices in split order, rounds (which is what the GEMM's own reduction does),
-// adds the residual and normalises.  NJ = 16-byte items per thread.
+// per row, as many threads as the row has 16-byte items (up to 512, then NJ = 2 items per thread),
+// adds the slices in split order, rounds (which is what the GEMM's own reduction does), adds the
+// residual and normalises.  Everything that does not depend on the sums is requested first.
 template <typename T, int NJ>
-__global__ __launch_bounds__(256) void ksa_add_rmsnorm_partials_kernel(const NormParams p) {
+__global__ __launch_bounds__(512) void ksa_add_rmsnorm_partials_kernel(const NormParams p) {
     using C = KsaCvt<T>;
-    __shared__ float s_ss[4];
-    const int tid = threadIdx.x;
+    __shared__ float s_ss[8];
+    const int tid = threadIdx.x, nthr = blockDim.x;
     const int row = blockIdx.x;
     const int items = p.H / 8;
-    u32x4 r[NJ], wv[NJ];
+    u32x4 r[NJ], wv[NJ], q[NJ];
     float ss = 0.f;
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) {  // the weights do not wait for the mean square
-        const int idx = tid + 256 * j;
-        if (idx < items) wv[j] = *reinterpret_cast<const u32x4*>(p.w + 8 * idx);
+    for (int j = 0; j < NJ; ++j) {  // the weights and the residual do not wait for the sums
+        const int idx = tid + nthr * j;
+        if (idx < items) {
+            wv[j] = *reinterpret_cast<const u32x4*>(p.w + 8 * idx);
+            q[j] = *reinterpret_cast<const u32x4*>(p.res + (int64_t)row * p.rs + 8 * idx);
+        }
     }
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
-        const int idx = tid + 256 * j;
+        const int idx = tid + nthr * j;
         if (idx < items) {
-            float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-            for (int sp0 = 0; sp0 < p.ksplit; sp0 += 8) {  // eight slices requested together
-                f32x4 lo[8], hi[8];
-#pragma unroll
-                for (int u = 0; u < 8; ++u) {
-                    const int sp = min(sp0 + u, p.ksplit - 1);
-                    const float* src = p.part + ((int64_t)sp * 16 + row) * p.H + 8 * idx;
-                    lo[u] = *reinterpret_cast<const f32x4*>(src);
-                    hi[u] = *reinterpret_cast<const f32x4*>(src + 4);
-                }
-#pragma unroll
-                for (int u = 0; u < 8; ++u) {
-                    if (sp0 + u < p.ksplit) {
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) acc[i] += lo[u][i], acc[4 + i] += hi[u][i];
-                    }
-                }
-            }
-            const u32x4 q = *reinterpret_cast<const u32x4*>(p.res + (int64_t)row * p.rs + 8 * idx);
+            const u32x4 x = ksa_sum_partials8<T>(p.part, p.ksplit, p.H, row, 8 * idx);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const uint32_t x2 = C::down2(acc[2 * i], acc[2 * i + 1]);
-                r[j][i] = C::down2(C::lo(x2) + C::lo(q[i]), C::hi(x2) + C::hi(q[i]));
+                r[j][i] = C::down2(C::lo(x[i]) + C::lo(q[j][i]), C::hi(x[i]) + C::hi(q[j][i]));
                 const float a = C::lo(r[j][i]), b = C::hi(r[j][i]);
                 ss = fmaf(a, a, ss);
                 ss = fmaf(b, b, ss);
@@ -136,11 +121,12 @@ __global__ __launch_bounds__(256) void ksa_add_rmsnorm_partials_kernel(const Nor
     for (int m = 32; m >= 1; m >>= 1) ss += __shfl_xor(ss, m);
     if ((tid & 63) == 0) s_ss[tid >> 6] = ss;
     __syncthreads();
-    ss = (s_ss[0] + s_ss[1]) + (s_ss[2] + s_ss[3]);
+    ss = 0.f;
+    for (int w = 0; w < nthr / 64; ++w) ss += s_ss[w];
     const float inv = rsqrtf(ss / (float)p.H + p.eps);
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
-        const int idx = tid + 256 * j;
+        const int idx = tid + nthr * j;
         if (idx < items) {
             u32x4 o;
 #pragma unroll
@@ -155,11 +141,12 @@ __global__ __launch_bounds__(256) void ksa_add_rmsnorm_partials_kernel(const Nor
 
 template <typename T>
 int dispatch_norm_partials(const NormParams& p, hipStream_t st) {
-    const int need = (p.H / 8 + 255) / 256;
-    const dim3 grid((unsigned)p.rows), block(256);
+    const int items = p.H / 8;
+    const int threads = items >= 512 ? 512 : (items + 63) / 64 * 64;
+    const int need = (items + threads - 1) / threads;
+    const dim3 grid((unsigned)p.rows), block(threads);
     if (need <= 1) hipLaunchKernelGGL((ksa_add_rmsnorm_partials_kernel<T, 1>), grid, block, 0, st, p);
     else if (need <= 2) hipLaunchKernelGGL((ksa_add_rmsnorm_partials_kernel<T, 2>), grid, block, 0, st, p);
-    else if (need <= 4) hipLaunchKernelGGL((ksa_add_rmsnorm_partials_kernel<T, 4>), grid, block, 0, st, p);
     else return KSA_ERR_UNSUPPORTED;
     return ksa_check_launch();
 }
