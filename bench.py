@@ -181,10 +181,6 @@ def main():
     ap.add_argument("--sustain", type=float, default=0.0, metavar="SECONDS",
                     help="also loop the prefill launch for SECONDS and report the rate of the second "
                          "half under 'sustained' (the chip lowers its clock under a long MFMA load)")
-    ap.add_argument("--mfma-ceiling", type=float, default=0.0, metavar="SECONDS",
-                    help="also time a pure bf16 MFMA instruction stream for SECONDS with random and "
-                         "with all-zero operands (second-half rate, 'mfma_stream'): the rate the "
-                         "power limit allows, to read the prefill rate against")
     ap.add_argument("--e2e", action="store_true",
                     help="also run the end-to-end decoder (random-init 4B shape: 36 layers, 3 Summary : 1 "
                          "full, batch 8, 32k-token prompt, 256 greedy steps) and report prefill and "
@@ -275,23 +271,6 @@ def main():
                                    "frac_of_peak": rate / PEAK_BF16_TFLOPS, "sclk_mhz_mean": clk}
         del q, k, v, sp
         torch.cuda.empty_cache()
-
-    if args.mfma_ceiling > 0:
-        import ctypes
-        L = _lib.lib()
-        out = torch.empty(256 * 8 * 64, dtype=torch.float32, device=dev)
-        fl = ctypes.c_double(0.0)
-        res = {}
-        for name, zero in (("random_operands", 0), ("zero_operands", 1)):
-            def mstep():
-                _lib.check(L.ksa_probe_mfma_stream(out.data_ptr(), 256, 8, 2000, zero, ctypes.byref(fl),
-                                                   _lib.stream_ptr(dev)), "ksa_probe_mfma_stream")
-            mstep()
-            torch.cuda.synchronize()
-            rate, clk = sustained_rate(mstep, fl.value, args.mfma_ceiling, 10)
-            res[name] = {"tflops_second_half": rate, "frac_of_peak": rate / PEAK_BF16_TFLOPS,
-                         "sclk_mhz_mean": clk}
-        result["mfma_stream"] = {"seconds_each": args.mfma_ceiling, "waves_per_simd": 2, **res}
 
     # ------------------------------------------------------------------ decode
     if not args.skip_decode:

@@ -8,7 +8,8 @@
  *
  * Conventions
  *   - every pointer is a DEVICE pointer owned by the caller unless stated otherwise;
- *     the library never allocates, frees or synchronises;
+ *     the library never allocates, frees or synchronises, keeps no state between calls and
+ *     reads no environment variable;
  *   - `stream` is a hipStream_t passed as void* (0 = the null stream);
  *   - 16-bit tensors are described by element strides; pointers must be 16-byte
  *     aligned and strides multiples of 8 elements, the innermost (head_dim) stride is 1;
@@ -66,13 +67,21 @@ int ksa_block_index(int Sq, int Sk, int C, int S, int W, int P, int skip_old, in
  *       rows * row stride * 2 bytes must stay below 4 GiB.
  *   out [batch, Sq, Hq, D]; lse fp32 [batch, Hq, Sq] (natural log) or NULL.
  *   mask_cnt .. full_idx: output of ksa_block_index(Sq, Sq+P, ..., 128, 64), idx_stride = N.
- *   scale: soft-max scale (the reference uses head_dim^-0.5). */
+ *   scale: soft-max scale (the reference uses head_dim^-0.5).
+ *   shape: workgroup shape, a tuning knob with no effect on the result beyond the tolerance of
+ *       the tests.  KSA_PREFILL_SHAPE_AUTO lets the library choose from the launch size and the
+ *       device's CU count; the others apply to head_dim 128 with an even Hq / Hkv and fall back
+ *       to one head per workgroup elsewhere. */
+#define KSA_PREFILL_SHAPE_AUTO 0       /* library's choice */
+#define KSA_PREFILL_SHAPE_1HEAD 32     /* one query head on 4 waves, 32 rows per wave */
+#define KSA_PREFILL_SHAPE_2HEAD_64 64  /* two heads of a kv group on 4 waves, 64 rows per wave */
+#define KSA_PREFILL_SHAPE_2HEAD 2      /* two heads of a kv group on 8 waves, 32 rows per wave */
 int ksa_prefill_fwd(const void* q, const void* k, const void* v, void* out, float* lse, int batch,
                     int Sq, int Hq, int Hkv, int D, int dtype, const int64_t* q_strides,
                     const int64_t* kv_strides, const int64_t* out_strides, int C, int S, int W,
                     int P, int skip_old, int phys_prefix, const int32_t* mask_cnt,
                     const int32_t* mask_idx, const int32_t* full_cnt, const int32_t* full_idx,
-                    int idx_stride, float scale, void* stream);
+                    int idx_stride, float scale, int shape, void* stream);
 
 /* Decode attention over the ring-buffer slice.
  * Replaces HF:591-612 (_sdpa_attention_forward, incl. repeat_kv :557-566) applied to the
@@ -190,14 +199,6 @@ size_t ksa_gemm_rows_workspace_bytes(int N, int ksplit);
 int ksa_gemm_rows(const void* x, const void* w, void* out, int M, int N, int K, long long x_row_stride,
                   long long w_row_stride, long long out_row_stride, int dtype, int ksplit,
                   void* workspace, size_t workspace_bytes, void* stream);
-
-/* Measurement aid (no counterpart in the reference): launches a pure stream of bf16 MFMA
- * 32x32x16 instructions (blocks x waves_per_block waves, 16 * iters instructions each, operands
- * random or all zero) and returns the floating-point operations of the launch in *flop.  Timed
- * over seconds it gives the MFMA rate the chip sustains under its power limit, against which
- * the prefill kernel's rate can be read.  out: device float[blocks * waves_per_block * 64]. */
-int ksa_probe_mfma_stream(void* out, int blocks, int waves_per_block, int iters,
-                          int zero_operands, double* flop, void* stream);
 
 /* Host-side diagnostic: number of key columns in [a, b) visible to query row q under the
  * closed-form rule the kernels use (no GPU involved). */

@@ -23,7 +23,7 @@ _SIGNATURES = {
     "ksa_device_cu_count": (_int, []),
     "ksa_block_index": (_int, [_int] * 9 + [_vp] * 4 + [_vp]),
     "ksa_prefill_fwd": (_int, [_vp] * 5 + [_int] * 6 + [_i64p] * 3 + [_int] * 6 + [_vp] * 4
-                        + [_int, ctypes.c_float, _vp]),
+                        + [_int, ctypes.c_float, _int, _vp]),
     "ksa_decode_workspace_bytes": (ctypes.c_size_t, [_int] * 6),
     "ksa_decode_auto_splits": (_int, [_int] * 3),
     "ksa_decode_fwd": (_int, [_vp] * 6 + [_int] * 8 + [_i64p] * 4
@@ -41,7 +41,6 @@ _SIGNATURES = {
     "ksa_gemm_rows_auto_splits": (_int, [_int, _int]),
     "ksa_gemm_rows_workspace_bytes": (ctypes.c_size_t, [_int, _int]),
     "ksa_gemm_rows": (_int, [_vp] * 3 + [_int] * 3 + [ctypes.c_longlong] * 3 + [_int, _int, _vp, ctypes.c_size_t, _vp]),
-    "ksa_probe_mfma_stream": (_int, [_vp] + [_int] * 4 + [ctypes.POINTER(ctypes.c_double), _vp]),
     "ksa_debug_count_visible": (ctypes.c_longlong, [ctypes.c_longlong] * 3 + [_int] * 7),
 }
 

@@ -20,8 +20,5 @@ extern "C" const char* ksa_error_string(int code) {
 
 // Number of compute units of the current device (0 if no device is usable).
 extern "C" int ksa_device_cu_count(void) {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess) return 0;
-    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
-    return n;
+    return ksa_cu_count_or(0);
 }

@@ -19,3 +19,12 @@ enum { KSA_DTYPE_BF16 = 0, KSA_DTYPE_F16 = 1 };
 static inline int ksa_check_launch() {
     return hipGetLastError() == hipSuccess ? KSA_OK : KSA_ERR_LAUNCH;
 }
+
+// Compute units of the current device, or `fallback` when no device can be asked (host-only use
+// of the heuristics).
+static inline int ksa_cu_count_or(int fallback) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return fallback;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return fallback;
+    return n;
+}

@@ -311,12 +311,13 @@ extern "C" size_t ksa_decode_workspace_bytes(int batch, int Hq, int Hkv, int Q, 
     return (size_t)batch * Hkv * nsplit * cols * (D + 2) * sizeof(float);
 }
 
-// Heuristic number of splits: at least two workgroups per CU (256 CUs), but never splits
-// shorter than 256 rows.
+// Heuristic number of splits: at least two workgroups per CU of the current device (256 CUs
+// assumed when no device can be asked), but never splits shorter than 256 rows.
 extern "C" int ksa_decode_auto_splits(int batch, int Hkv, int max_rows) {
     if (batch <= 0 || Hkv <= 0 || max_rows <= 0) return 1;
     const int units = batch * Hkv;
-    int n = (512 + units - 1) / units;
+    const int want = 2 * ksa_cu_count_or(256);
+    int n = (want + units - 1) / units;
     const int cap = max_rows / 256 > 1 ? max_rows / 256 : 1;
     if (n > cap) n = cap;
     if (n > 64) n = 64;

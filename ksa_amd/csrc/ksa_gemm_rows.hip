@@ -133,14 +133,16 @@ int launch_gemm(const GemmParams& p, hipStream_t st) {
 
 }  // namespace
 
-// K splits that give about two workgroups per CU (256 CUs) without slices shorter than one chunk
+// K splits that give about two workgroups per CU of the current device (256 CUs assumed when no
+// device can be asked) without slices shorter than one chunk
 // of 512; when one chunk per workgroup is at least that many splits and still a moderate grid,
 // that is taken instead: a workgroup then stages x once and has no loop (measured 11 % faster at
 // N = 19456, K = 2560).
 extern "C" int ksa_gemm_rows_auto_splits(int N, int K) {
     if (N <= 0 || K <= 0) return 1;
     const int tiles = (N + 63) / 64;
-    int sp = (512 + tiles - 1) / tiles;
+    const int want = 2 * ksa_cu_count_or(256);
+    int sp = (want + tiles - 1) / tiles;
     const int chunks = K / 32 / 16 > 1 ? K / 32 / 16 : 1;
     if (sp > chunks) sp = chunks;
     if (sp > 16) sp = 16;

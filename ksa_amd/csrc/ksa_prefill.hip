@@ -36,7 +36,6 @@
 // the workgroup repeats the walk with the textbook online soft-max.
 #include <hip/hip_runtime.h>
 #include <math.h>
-#include <stdlib.h>
 
 #include <type_traits>
 
@@ -66,7 +65,7 @@ struct PrefillParams {
     KsaMask mk;
     float scale;
     float scale_log2;
-    int shape;  // 0: default; 32: one head per workgroup; 64: two heads, 64 query rows per wave
+    int shape;  // 2: two heads on 8 waves; 32: one head per workgroup; 64: two heads, 64 query rows per wave
 };
 
 constexpr int kTileM = 128;
@@ -676,8 +675,15 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
 #pragma unroll
         for (int r = 0; r < RB; ++r) {
             const float l_tot = ksa_pair_sum(l_run[r]);
-            // every row sees at least itself: a vanishing sum means a reference far too high
-            bad = bad || !(l_tot > 5.4e-20f);
+            // Every row sees at least itself: a small sum means a reference far too high.  How
+            // small depends on what the 16-bit probabilities can hold.  bf16 has fp32's exponent
+            // range, so only a vanishing sum (below 2^-64) loses anything.  fp16 is exact in
+            // relative terms down to 2^-14 and absolute (steps of 2^-24) below: with a row sum
+            // of at least 2^-4 the rounding of n probabilities adds up to at most n 2^-25 / 2^-4
+            // of the sum (2^-8 for 8192 keys, in practice its square root); below that the row
+            // is walked again with exact references.
+            constexpr float kMinRowSum = std::is_same<T, KsaF16>::value ? 0.0625f : 5.4e-20f;
+            bad = bad || !(l_tot > kMinRowSum);
         }
         if (__syncthreads_or(bad)) walk(std::true_type{});
     }
@@ -727,7 +733,7 @@ int launch(const PrefillParams& p, int batch, hipStream_t stream) {
     if constexpr (D == 128) {
         if (p.g % 2 == 0) {
             if (p.shape == 64) return launch_shape<T, D, 2, 2>(p, batch, stream);
-            if (p.shape != 32) return launch_shape<T, D, 1, 2>(p, batch, stream);
+            if (p.shape == 2) return launch_shape<T, D, 1, 2>(p, batch, stream);
         }
     }
     return launch_shape<T, D, 1, 1>(p, batch, stream);
@@ -744,13 +750,15 @@ extern "C" int ksa_prefill_fwd(const void* q, const void* k, const void* v, void
                                const int64_t* out_strides, int C, int S, int W, int P,
                                int skip_old, int phys_prefix, const int32_t* mask_cnt,
                                const int32_t* mask_idx, const int32_t* full_cnt,
-                               const int32_t* full_idx, int idx_stride, float scale, void* stream) {
+                               const int32_t* full_idx, int idx_stride, float scale, int shape,
+                               void* stream) {
     if (!q || !k || !v || !out || !mask_cnt || !mask_idx || !full_cnt || !full_idx) return KSA_ERR_NULL;
     if (!q_strides || !kv_strides || !out_strides) return KSA_ERR_NULL;
     if (batch <= 0 || Sq <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0) return KSA_ERR_INVALID;
     if (C <= 0 || S <= 0 || W < 0 || P < 0) return KSA_ERR_INVALID;
     if ((int64_t)Sq + P >= (1ll << 30)) return KSA_ERR_INVALID;
     if (dtype != KSA_DTYPE_BF16 && dtype != KSA_DTYPE_F16) return KSA_ERR_UNSUPPORTED;
+    if (shape != 0 && shape != 2 && shape != 32 && shape != 64) return KSA_ERR_INVALID;
     const int Sk = Sq + P;
     const int N = (Sk + kTileN - 1) / kTileN;
     if (idx_stride < N) return KSA_ERR_INVALID;
@@ -792,13 +800,12 @@ extern "C" int ksa_prefill_fwd(const void* q, const void* k, const void* v, void
     p.scale = scale;
     p.scale_log2 = scale * 1.4426950408889634f;
     // Workgroup shape (D = 128, even group size; anything else uses one head per workgroup):
-    // default two heads on 8 waves; KSA_PREFILL_ROWS_PER_WAVE=32 (or a short launch) one head on 4 waves;
-    // =64 two heads on 4 waves with 64 query rows per wave (one wave per SIMD).
-    // A short launch (fewer than 16 two-head workgroups per CU of the 256) takes the one-head shape:
-    // two of its workgroups share a CU and hide each other's start and end (8k rows: +9 %,
-    // 16k: +4 %, 24k: +1.5 %, 32k rows and up: the same within 1 %).
-    const char* rpw = getenv("KSA_PREFILL_ROWS_PER_WAVE");
-    p.shape = rpw ? atoi(rpw) : ((int64_t)p.M * (Hq / 2) * batch < 16 * 256 ? 32 : 0);
+    // 2 = two heads on 8 waves; 32 = one head on 4 waves; 64 = two heads on 4 waves with 64 query
+    // rows per wave (one wave per SIMD).  Left to the library (0), a short launch (fewer than 16
+    // two-head workgroups per CU of the device) takes the one-head shape: two of its workgroups
+    // share a CU and hide each other's start and end (8k rows: +9 %, 16k: +4 %, 24k: +1.5 %,
+    // 32k rows and up: the same within 1 %); longer launches take two heads on 8 waves.
+    p.shape = shape ? shape : ((int64_t)p.M * (Hq / 2) * batch < 16ll * ksa_cu_count_or(256) ? 32 : 2);
 
     hipStream_t st = (hipStream_t)stream;
     if (dtype == KSA_DTYPE_BF16) {

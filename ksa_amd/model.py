@@ -19,8 +19,11 @@ Differences from the reference, on purpose:
   this package's kernels;
 * a "full attention" layer is, as in the reference's inference model, a Summary layer whose
   window is larger than any sequence (append-only text cache, :114-115, :232-242);
-* `summary_independent_parameters` is supported for mix_coeff 0 and 1 (the reference's default
-  1.0, :765-791): the summary rows then take their q, k, v from their own projection.
+* `summary_independent_parameters` (:756-789): for mix_coeff 1 (the reference's default) the
+  summary rows take their q, k, v from their own projection, for mix_coeff 0 that projection is
+  unused, and in between the two are blended.  The reference blends the normalised q and k (and
+  the plain v) before the rotary embedding; the rotation is linear, so the blend is done here on
+  the outputs of the fused pre-attention step instead.
 
 The attention-side and element-wise operators come from an `ops` object; the default binds the
 HIP kernels of this package and needs a GPU.  Tests pass a CPU fp32 implementation of the same
@@ -221,8 +224,8 @@ class KsaQwen3ForCausalLM:
         self.config = config
         self.w = weights
         self.ops = ops if ops is not None else HipOps()
-        if config.summary_independent_parameters and config.mix_coeff not in (0, 0.0, 1, 1.0):
-            raise NotImplementedError("summary_independent_parameters needs mix_coeff 0 or 1")
+        if config.summary_independent_parameters and not 0.0 <= float(config.mix_coeff) <= 1.0:
+            raise ValueError("mix_coeff must lie in [0, 1]")
         self.scns = config.sliding_chunk_nums()
         D = config.head_dim
         self.inv_freq = 1.0 / (config.rope_theta ** (torch.arange(0, D, 2, dtype=torch.int64).float() / D))
@@ -230,7 +233,6 @@ class KsaQwen3ForCausalLM:
         emb = weights["embed_tokens"]
         self.dtype, self.device = emb.dtype, emb.device
         self.inv_freq_dev = self.inv_freq.to(self.device)
-        self._graphs = {}
         self.lm_head = emb[: config.vocab_size] if config.tie_word_embeddings else weights["lm_head"]
 
     # ---- pieces ----------------------------------------------------------------------
@@ -251,10 +253,25 @@ class KsaQwen3ForCausalLM:
         cfg = self.config
         D, Hq, Hkv = cfg.head_dim, cfg.num_attention_heads, cfg.num_key_value_heads
         qkv = self.ops.linear(h, lw["qkv_proj"])
-        if (cfg.summary_independent_parameters and cfg.mix_coeff != 0 and summary_rows is not None
+        if (cfg.summary_independent_parameters and cfg.mix_coeff == 1 and summary_rows is not None
                 and summary_rows.numel() > 0):
             qkv[:, summary_rows] = self.ops.linear(h[:, summary_rows], lw["qkv_proj_summary"])
         return self._split_qkv(qkv)
+
+    def _blend_summary(self, lw, h, summary_rows, cos, sin, q, k, v):
+        """mix_coeff strictly between 0 and 1 (:776-788): the summary rows of q, k, v (already
+        normalised and rotated, from the shared projection) become
+        mix * (the same from the summary projection) + (1 - mix) * themselves, in place."""
+        cfg = self.config
+        m = float(cfg.mix_coeff)
+        if (not cfg.summary_independent_parameters or m in (0.0, 1.0) or summary_rows is None
+                or summary_rows.numel() == 0):
+            return
+        qs, ks, vs = self._split_qkv(self.ops.linear(h[:, summary_rows], lw["qkv_proj_summary"]))
+        qs, ks, vs = self.ops.pre_attention(qs, ks, vs, lw["q_norm"], lw["k_norm"], cos[:, summary_rows],
+                                            sin[:, summary_rows], cfg.rms_norm_eps)
+        for dst, src in ((q, qs), (k, ks), (v, vs)):
+            dst[:, summary_rows] = (m * src + (1.0 - m) * dst[:, summary_rows]).to(dst.dtype)
 
     def _split_qkv(self, qkv):
         cfg = self.config
@@ -295,6 +312,7 @@ class KsaQwen3ForCausalLM:
             k_slot, v_slot = cache.prefill_slots(li, b, Hkv, L, D, self.dtype, self.device, n_sum)
             q, k, v = ops.pre_attention(q, k, v, lw["q_norm"], lw["k_norm"], cos, sin, cfg.rms_norm_eps,
                                         k_out=k_slot, v_out=v_slot)
+            self._blend_summary(lw, h, sum_rows, cos, sin, q, k, v)
             attn, _ = ops.summary_attn_func(q, k, v, C, S, self.scns[li], summary_pos=is_sum)
             x, h = self._add_norm(ops.linear(attn.reshape(b, L, -1), lw["o_proj"]), x, lw["post_attention_layernorm"])
             delta = self._mlp(lw, h)
@@ -345,6 +363,7 @@ class KsaQwen3ForCausalLM:
             else:
                 q, k, v = self._qkv(lw, h, sum_rows)
                 q, k, v = ops.pre_attention(q, k, v, lw["q_norm"], lw["k_norm"], cos, sin, cfg.rms_norm_eps)
+                self._blend_summary(lw, h, sum_rows, cos, sin, q, k, v)
                 qh, kh, vh = q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2)
                 cache.update_text(kh[:, :, :1], vh[:, :, :1], li)
                 a, e = cache.attention_range(li)
@@ -398,7 +417,9 @@ class KsaQwen3ForCausalLM:
     def decode_step_graph(self, token_ids: torch.Tensor, cache):
         """`decode_step` with the launches of a non-boundary step replayed from a HIP graph (about
         400 launches per step otherwise cost more host time than GPU time).  Chunk-boundary steps
-        run as in `decode_step`.  The graph is recorded again when a cache buffer was reallocated.
+        run as in `decode_step`.  The recording belongs to the cache object it was made for (it is
+        kept on it) and is made again when a cache buffer was reallocated or changed its shape:
+        the launches bake in the buffers' addresses, strides and capacity.
         The returned logits live in a buffer that the next call overwrites."""
         cfg = self.config
         C, S = cfg.summary_chunk_size, cfg.summary_token_num
@@ -406,14 +427,14 @@ class KsaQwen3ForCausalLM:
             return self.decode_step(token_ids, cache)
         b = token_ids.shape[0]
         Hkv, D = cfg.num_key_value_heads, cfg.head_dim
-        st = self._graphs.get(id(cache))
-        if st is None or st["batch"] != b:
-            st = {"batch": b, "graph": None, "ptrs": None,
+        st = getattr(cache, "_ksa_graph_state", None)
+        if st is None or st["batch"] != b or st["owner"] is not self:
+            st = {"batch": b, "owner": self, "graph": None, "ptrs": None,
                   "tok": torch.zeros(b, 1, dtype=torch.long, device=self.device),
                   "pos": torch.zeros(1, 1, dtype=torch.long, device=self.device),
                   # [kind: small / large window][destination row, range start, range end][sequence]
                   "cur": torch.zeros(2, 3, b, dtype=torch.int32, device=self.device)}
-            self._graphs = {id(cache): st}
+            cache._ksa_graph_state = st
         p = cache.get_true_token_num() if cfg.summary_chunk_position_ids_type == "origin" \
             else cache.get_cur_chunk_size()
         # host bookkeeping of the step (may enlarge an append-only buffer), then this step's rows
@@ -435,7 +456,7 @@ class KsaQwen3ForCausalLM:
         st["cur"].copy_(torch.tensor(vals, dtype=torch.int32).view(2, 3, 1))
         st["tok"].copy_(token_ids.to(self.device))
         st["pos"].fill_(p)
-        ptrs = tuple(t.data_ptr() for t in cache.key_cache + cache.value_cache)
+        ptrs = tuple((t.data_ptr(), tuple(t.shape), t.stride()) for t in cache.key_cache + cache.value_cache)
         if st["graph"] is None or st["ptrs"] != ptrs:
             side = torch.cuda.Stream(device=self.device)
             side.wait_stream(torch.cuda.current_stream(self.device))

@@ -10,7 +10,6 @@ libksa_hip.so; there is no other execution path.
 from __future__ import annotations
 
 import ctypes
-import weakref
 from typing import Dict, Optional, Tuple
 
 import torch
@@ -27,6 +26,12 @@ TILE_N = 64
 SUMMARY_ATTN_CACHE: Dict[Tuple, Tuple[torch.Tensor, ...]] = {}
 
 _DTYPES = {torch.bfloat16: 0, torch.float16: 1}
+
+# Workgroup shape handed to ksa_prefill_fwd when a call does not name one: 0 = the library's
+# choice, 2 = two heads on 8 waves, 32 = one head on 4 waves, 64 = two heads on 4 waves with 64
+# query rows per wave (include/ksa_hip.h, KSA_PREFILL_SHAPE_*).  A tuning knob: results agree to
+# the tolerance of the tests, only the speed differs.
+PREFILL_SHAPE = 0
 
 
 class BlockSparseIndex(tuple):
@@ -69,20 +74,39 @@ def _cached_index(Sq, C, S, W, P, skip_old, device) -> BlockSparseIndex:
     return idx
 
 
-# summary_pos analysis is cached per tensor object (HF passes the same mask to every layer)
-# id(tensor) -> (weakref to it, version, (Sq, C, S), result)
-_POS_CACHE: Dict[int, tuple] = {}
+# summary_pos analysis is cached per buffer: the HF call site hands every layer a fresh
+# `summary_mask.squeeze(0)` view of one tensor (modeling_qwen3sa.py:807-815), so the key is the
+# storage address, not the Python object.
+# An entry holds the tensor it analysed, which keeps that storage alive: while the entry exists
+# the address cannot be handed to another mask.
+# (data_ptr, numel, device, Sq, C, S) -> (tensor, version or None, result)
+_POS_CACHE: Dict[tuple, tuple] = {}
+_POS_CACHE_MAX = 16
+_POS_ANALYSES = 0   # number of analyses actually run (each costs one host synchronisation)
+
+
+def _pos_version(t: torch.Tensor):
+    """In-place modification counter of `t`, or None for inference tensors, which have none
+    (reading `_version` on them raises)."""
+    return None if t.is_inference() else t._version
 
 
 def _analyse_summary_pos(summary_pos: torch.Tensor, Sq: int, C: int, S: int):
     """Returns (P, periodic, rows): P = number of summary rows; periodic = summary_pos
     is exactly `(i % (C+S)) >= C` over whole blocks followed by text rows only, so that
     prefix row j can be read in place at (j//S)*(C+S)+C+j%S; rows = int32 row indices of
-    the summary rows (only when not periodic)."""
-    hit = _POS_CACHE.get(id(summary_pos))
-    ver = summary_pos._version
-    if hit is not None and hit[0]() is summary_pos and hit[1] == ver and hit[2] == (Sq, C, S):
-        return hit[3]
+    the summary rows (only when not periodic).
+
+    The result is kept per (storage address, length, device, Sq, C, S) together with the
+    tensor's in-place modification counter.  Inference tensors have no such counter: a mask made
+    under torch.inference_mode() and later rewritten in place must be followed by
+    `clear_summary_pos_cache()`."""
+    global _POS_ANALYSES
+    key = (summary_pos.data_ptr(), summary_pos.numel(), str(summary_pos.device), Sq, C, S)
+    ver = _pos_version(summary_pos)
+    hit = _POS_CACHE.get(key)
+    if hit is not None and hit[1] == ver:
+        return hit[2]
     if summary_pos.dtype != torch.bool or summary_pos.dim() != 1 or summary_pos.numel() != Sq:
         raise AssertionError("summary_pos must be a bool tensor of shape [seqlen_q]")
     B = C + S
@@ -97,10 +121,15 @@ def _analyse_summary_pos(summary_pos: torch.Tensor, Sq: int, C: int, S: int):
     if not periodic:
         rows = torch.nonzero(summary_pos, as_tuple=False).flatten().to(torch.int32)
     res = (P, periodic, rows)
-    if len(_POS_CACHE) > 64:
+    _POS_ANALYSES += 1
+    if len(_POS_CACHE) >= _POS_CACHE_MAX:
         _POS_CACHE.clear()
-    _POS_CACHE[id(summary_pos)] = (weakref.ref(summary_pos), ver, (Sq, C, S), res)
+    _POS_CACHE[key] = (summary_pos, ver, res)
     return res
+
+
+def clear_summary_pos_cache() -> None:
+    _POS_CACHE.clear()
 
 
 def _check_inputs(q, k, v):
@@ -125,7 +154,8 @@ def _lastdim_contig(t):
 def _summary_attn_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
                       mask_cnt: torch.Tensor, mask_idx: torch.Tensor, full_cnt: torch.Tensor,
                       full_idx: torch.Tensor, C: int, S: int, W: int, P: int, skip_old: bool,
-                      phys_prefix: bool, scale: float, want_lse: bool) -> Tuple[torch.Tensor, torch.Tensor]:
+                      phys_prefix: bool, scale: float, want_lse: bool,
+                      shape: int) -> Tuple[torch.Tensor, torch.Tensor]:
     b, Sq, Hq, D = q.shape
     Hkv = k.shape[2]
     out = torch.empty_like(q)
@@ -139,14 +169,14 @@ def _summary_attn_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
             _lib.strides3(q, dims), _lib.strides3(k, dims), _lib.strides3(out, dims),
             C, S, W, P, int(skip_old), int(phys_prefix),
             mask_cnt.data_ptr(), mask_idx.data_ptr(), full_cnt.data_ptr(), full_idx.data_ptr(),
-            mask_idx.shape[-1], float(scale), _lib.stream_ptr(q.device))
+            mask_idx.shape[-1], float(scale), int(shape), _lib.stream_ptr(q.device))
     _lib.check(rc, "ksa_prefill_fwd")
     return out, lse
 
 
 @_summary_attn_fwd.register_fake
 def _(q, k, v, mask_cnt, mask_idx, full_cnt, full_idx, C, S, W, P, skip_old, phys_prefix, scale,
-      want_lse):
+      want_lse, shape):
     b, Sq, Hq, _ = q.shape
     return torch.empty_like(q), q.new_empty((b, Hq, Sq) if want_lse else (0,), dtype=torch.float32)
 
@@ -171,7 +201,7 @@ def _gathered_prefix(t: torch.Tensor, rows: torch.Tensor, P: int) -> torch.Tenso
 def summary_attn_func(q, k, v, chunk_size, summary_num, sliding_chunk_num,
                       summary_pos: Optional[torch.Tensor] = None,
                       skip_old_summary: bool = False, *, return_lse: bool = False,
-                      softmax_scale: Optional[float] = None):
+                      softmax_scale: Optional[float] = None, workgroup_shape: Optional[int] = None):
     """q [b, Sq, Hq, D]; k, v [b, Sq (+P), Hkv, D]; returns (out [b, Sq, Hq, D], lse or None).
 
     With `summary_pos` (bool [Sq]) the summary rows of k/v form the key prefix, as
@@ -181,8 +211,9 @@ def summary_attn_func(q, k, v, chunk_size, summary_num, sliding_chunk_num,
     a [prefix | in-line] buffer first.  Without `summary_pos`, the first
     `k.shape[1] - q.shape[1]` rows of k/v are taken as an already-built prefix.
     Forward only: tensors that require grad under an enabled grad mode are rejected.
-    `return_lse` / `softmax_scale` are extensions (the reference returns lse only for
-    autograd and always uses head_dim ** -0.5).
+    `return_lse` / `softmax_scale` / `workgroup_shape` are extensions (the reference returns lse
+    only for autograd and always uses head_dim ** -0.5; `workgroup_shape` is the tuning knob of
+    `PREFILL_SHAPE`).
     """
     _check_inputs(q, k, v)
     if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad):
@@ -209,5 +240,6 @@ def summary_attn_func(q, k, v, chunk_size, summary_num, sliding_chunk_num,
     scale = float(D) ** -0.5 if softmax_scale is None else float(softmax_scale)
     out, lse = torch.ops.ksa_amd.summary_attn_fwd(
         q, k, v, idx[0], idx[1], idx[2], idx[3], C, S, W, P,
-        bool(skip_old_summary), phys, scale, bool(return_lse))
+        bool(skip_old_summary), phys, scale, bool(return_lse),
+        PREFILL_SHAPE if workgroup_shape is None else int(workgroup_shape))
     return out, (lse if return_lse else None)

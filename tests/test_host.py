@@ -40,7 +40,7 @@ def test_error_codes_before_launch():
     assert L.ksa_block_index(100, 110, 128, 8, 3, 10, 0, 128, 64, None, None, None, None, None) == -2
     null3 = ctypes.cast(None, ctypes.POINTER(ctypes.c_int64))
     assert L.ksa_prefill_fwd(None, None, None, None, None, 1, 128, 4, 2, 128, 0, null3, null3, null3,
-                             128, 8, 3, 0, 0, 0, None, None, None, None, 2, 1.0, None) == -2
+                             128, 8, 3, 0, 0, 0, None, None, None, None, 2, 1.0, 0, None) == -2
     assert L.ksa_decode_fwd(None, None, None, None, None, None, 0, 10, 1, 4, 2, 1, 128, 0, null3, null3,
                             null3, null3, 1.0, 1, None, 0, None) == -2
     assert L.ksa_decode_workspace_bytes(64, 32, 8, 1, 128, 1) == 0
@@ -202,3 +202,37 @@ def test_split_heuristics_are_host_only_and_bounded():
     for b, h, rows in [(64, 8, 17288), (8, 8, 40000), (1, 1, 100), (1, 8, 1 << 20)]:
         assert 1 <= L.ksa_decode_auto_splits(b, h, rows) <= 64
     assert L.ksa_decode_auto_splits(64, 8, 17288) == 1
+
+
+def test_summary_pos_analysis_runs_once_for_fresh_views():
+    """The HF call site passes `summary_mask.squeeze(0)`, a new tensor object per layer
+    (modeling_qwen3sa.py:807-815): the analysis (one host synchronisation) must run once per
+    buffer, not once per view, also for masks made under torch.inference_mode(), whose tensors
+    have no modification counter."""
+    from ksa_amd import prefill
+    C, S = 16, 2
+    Sq = 5 * (C + S) + 7
+    for inference in (False, True):
+        prefill.clear_summary_pos_cache()
+        ctx = torch.inference_mode() if inference else torch.no_grad()
+        with ctx:
+            mask = (torch.arange(Sq) % (C + S) >= C)[None].clone()
+            mask[0, 5 * (C + S):] = False
+            before = prefill._POS_ANALYSES
+            res = [prefill._analyse_summary_pos(mask.squeeze(0), Sq, C, S) for _ in range(3)]
+        assert prefill._POS_ANALYSES - before == 1, inference
+        assert all(r is res[0] for r in res)
+        assert res[0][0] == 5 * S and res[0][1] is True and res[0][2] is None
+    # an in-place edit of a tracked tensor is seen
+    prefill.clear_summary_pos_cache()
+    mask = (torch.arange(Sq) % (C + S) >= C).clone()
+    mask[5 * (C + S):] = False
+    a = prefill._analyse_summary_pos(mask, Sq, C, S)
+    mask[3] = True
+    b = prefill._analyse_summary_pos(mask, Sq, C, S)
+    assert a[1] is True and b[1] is False and b[0] == a[0] + 1
+    assert b[2].tolist() == sorted([3] + [i for i in range(5 * (C + S)) if i % (C + S) >= C])
+    # a new mask of the same shape that reuses nothing of the old one is analysed on its own
+    other = torch.zeros(Sq, dtype=torch.bool)
+    assert prefill._analyse_summary_pos(other, Sq, C, S)[0] == 0
+    prefill.clear_summary_pos_cache()

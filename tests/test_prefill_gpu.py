@@ -89,16 +89,22 @@ def test_index_cfg2_known_answer():
     assert int((idx[0] + idx[2]).max()) == ka["W4"]["max_tiles_per_row_tile"]
 
 
-@pytest.fixture(params=["0", "32", "64", None], ids=["two_heads", "rows32", "rows64", "auto"])
+@pytest.mark.parametrize("W", [3, 4])
+def test_index_cfg2_bit_exact(W):
+    """cfg 2, the benchmark shape: all four index tensors (1088 x 2304 tiles) bit for bit against
+    the brute-force classifier of the C oracle, which evaluates the mask predicate on every one
+    of the 139264 x 147456 (query, key) pairs (about half a minute on 8 host threads)."""
+    _index_case(139264, 128, 8, W, 8192, False)
+
+
+@pytest.fixture(params=[2, 32, 64, 0], ids=["two_heads", "rows32", "rows64", "auto"])
 def wave_rows(request, monkeypatch):
-    """The workgroup shapes of the prefill kernel (D = 128, even group size): two heads on 8
-    waves (KSA_PREFILL_ROWS_PER_WAVE=0; what a long launch gets by default), one head on 4 waves
-    (=32; what a short launch gets by default) and two heads on 4 waves with 64 query rows per
-    wave (=64); unset = the library's own choice.  The library reads the variable on every call."""
-    if request.param is None:
-        monkeypatch.delenv("KSA_PREFILL_ROWS_PER_WAVE", raising=False)
-    else:
-        monkeypatch.setenv("KSA_PREFILL_ROWS_PER_WAVE", request.param)
+    """The workgroup shapes of the prefill kernel (D = 128, even group size), passed as the
+    `shape` argument of ksa_prefill_fwd: two heads on 8 waves (2; what a long launch gets from the
+    library), one head on 4 waves (32; what a short launch gets) and two heads on 4 waves with 64
+    query rows per wave (64); 0 = the library's own choice."""
+    import ksa_amd.prefill
+    monkeypatch.setattr(ksa_amd.prefill, "PREFILL_SHAPE", request.param)
     return request.param
 
 
@@ -319,8 +325,15 @@ def test_prefill_rejects_bad_inputs():
     with pytest.raises(AssertionError):
         ksa_amd.summary_attn_func(q, k, k, 128, 8, 1)
     q96 = torch.zeros(1, 136, 4, 96, device=dev, dtype=torch.bfloat16)
-    with pytest.raises(ksa_amd.KsaError):
+    # the reference takes any head_dim <= 256 that is a multiple of 8
+    # (flash_attn/cute/interface.py:206-208); this build has kernels for 64 and 128 only and says so
+    with pytest.raises(ksa_amd.KsaError, match=r"head_dim 64 or 128.*code -3"):
         ksa_amd.summary_attn_func(q96, q96, q96, 128, 8, 1)
+    q264 = torch.zeros(1, 136, 4, 264, device=dev, dtype=torch.bfloat16)
+    with pytest.raises(AssertionError, match="at most 256"):   # the reference's own rule
+        ksa_amd.summary_attn_func(q264, q264, q264, 128, 8, 1)
+    with pytest.raises(ksa_amd.KsaError, match=r"head_dim 64 or 128.*code -3"):
+        ksa_amd.ksa_decode(q96[:, :1].transpose(1, 2), q96.transpose(1, 2), q96.transpose(1, 2), 0, 136)
     qg = q.clone().requires_grad_(True)
     with pytest.raises(NotImplementedError):
         ksa_amd.summary_attn_func(qg, q, q, 128, 8, 1)
@@ -383,6 +396,30 @@ def test_prefill_reference_far_too_high(wave_rows):
     assert np.abs(lse[:, rows] - wlse).max() <= 0.1 + 1e-3 * np.abs(wlse).max()
 
 
+@pytest.mark.parametrize("boost", [3.0, 6.0, 10.0])
+def test_prefill_fp16_reference_moderately_too_high(boost, wave_rows):
+    """fp16 probabilities are exact in relative terms only down to 2^-14: a summary row whose
+    visible scores lie 7 to 20 octaves below the reference taken from the unmasked first tile
+    (summary keys it does not see, with a moderately larger norm) would keep a non-vanishing
+    but heavily quantised row sum.  The kernel has to redo such rows with exact references."""
+    Sq, Hq, Hkv, D, C, S, W = 24 * 136, 4, 2, 128, 128, 8, 2
+    q, k, v = make_qkv(Sq, Hq, Hkv, D, seed=10, scaled=False)
+    sp = O.summary_positions(Sq, C, S)
+    scale = torch.ones(Sq)
+    scale[torch.as_tensor(sp)] = boost
+    k = (k.float() * scale[:, None, None]).to(torch.float16)
+    q, v = q.to(torch.float16), v.to(torch.float16)
+    got, lse = _run_prefill(q, k, v, C, S, W, sp)
+    rows = np.r_[0:Sq:5].astype(np.int32)
+    rows = np.union1d(rows, np.nonzero(sp)[0]).astype(np.int32)   # every summary row
+    want, wlse = c_oracle.attention_rows(to_np(q), to_np(k), to_np(v), C, S, W, summary_pos=sp, rows=rows)
+    assert np.isfinite(got).all()
+    err = np.abs(got[rows] - want).max()
+    # fp16 carries 3 more mantissa bits than bf16: the bar is the bf16 one all the same
+    assert err <= ATOL * max(1.0, np.abs(want).max()), err
+    assert np.abs(lse[:, rows] - wlse).max() <= 2e-2 + 1e-3 * np.abs(wlse).max()
+
+
 @pytest.mark.parametrize("seed", [11, 12, 13])
 def test_prefill_random_shapes(seed, monkeypatch):
     """Twelve random small problems per seed - chunk sizes that are no power of two, summary
@@ -402,11 +439,7 @@ def test_prefill_random_shapes(seed, monkeypatch):
         mode = str(rng.choice(["prefix", "prefix", "inline", "physical"]))
         skip = bool(rng.integers(0, 2))
         dtype = torch.bfloat16 if rng.integers(0, 4) else torch.float16
-        shape = str(rng.choice(["", "0", "32", "64"]))
-        if shape:
-            monkeypatch.setenv("KSA_PREFILL_ROWS_PER_WAVE", shape)
-        else:
-            monkeypatch.delenv("KSA_PREFILL_ROWS_PER_WAVE", raising=False)
+        shape = int(rng.choice([0, 2, 32, 64]))
         q, k, v = make_qkv(Sq, Hq, Hkv, D, seed=seed * 100 + ci, scaled=bool(rng.integers(0, 2)))
         q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
         sp = O.summary_positions(Sq, C, S)
@@ -418,7 +451,8 @@ def test_prefill_random_shapes(seed, monkeypatch):
             st = torch.as_tensor(sp)
             kk, vv, spt = torch.cat([k[st], k]), torch.cat([v[st], v]), None
         out, lse = ksa_amd.summary_attn_func(q[None].to(dev), kk[None].to(dev), vv[None].to(dev), C, S, W,
-                                             summary_pos=spt, skip_old_summary=skip, return_lse=True)
+                                             summary_pos=spt, skip_old_summary=skip, return_lse=True,
+                                             workgroup_shape=shape)
         want, wlse = c_oracle.attention_rows(to_np(q), to_np(k), to_np(v), C, S, W, summary_pos=osp, skip_old=skip)
         got = to_np(out[0])
         assert np.isfinite(got).all(), case
