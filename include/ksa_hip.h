@@ -8,8 +8,9 @@
  *
  * Conventions
  *   - every pointer is a DEVICE pointer owned by the caller unless stated otherwise;
- *     the library never allocates, frees or synchronises, keeps no state between calls and
- *     reads no environment variable;
+ *     the library never allocates, frees or synchronises, keeps no state between calls (the one
+ *     exception, a fixed scratch array, is described at ksa_decode_fwd_noalloc) and reads no
+ *     environment variable;
  *   - `stream` is a hipStream_t passed as void* (0 = the null stream);
  *   - 16-bit tensors are described by element strides; pointers must be 16-byte
  *     aligned and strides multiples of 8 elements, the innermost (head_dim) stride is 1;
@@ -100,6 +101,24 @@ int ksa_decode_fwd(const void* q, const void* kcache, const void* vcache, void* 
                    int Hq, int Hkv, int Q, int D, int dtype, const int64_t* q_strides,
                    const int64_t* k_strides, const int64_t* v_strides, const int64_t* out_strides,
                    float scale, int nsplit, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ksa_decode_fwd for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
+ * Same arguments and results as ksa_decode_fwd without the workspace: the split-K partials go to
+ * a fixed array inside the library (KSA_DECODE_NOALLOC_SCRATCH_BYTES = 32 MiB of device memory
+ * per GPU the library runs on, held until the process ends).  The call allocates and frees
+ * nothing and does not synchronise.  A problem whose ksa_decode_workspace_bytes(...) exceeds
+ * ksa_decode_noalloc_max_workspace_bytes() is rejected with KSA_ERR_WORKSPACE before any launch.
+ * All calls on one GPU share the array: calls that overlap in time on one GPU (different
+ * streams or host threads) race and must be serialised by the caller; back-to-back calls on one
+ * stream are safe, nothing has to be cleared between them. */
+#define KSA_DECODE_NOALLOC_SCRATCH_BYTES (32u << 20)
+size_t ksa_decode_noalloc_max_workspace_bytes(void);
+int ksa_decode_fwd_noalloc(const void* q, const void* kcache, const void* vcache, void* out,
+                           const int32_t* start, const int32_t* end, int start0, int end0, int batch,
+                           int Hq, int Hkv, int Q, int D, int dtype, const int64_t* q_strides,
+                           const int64_t* k_strides, const int64_t* v_strides,
+                           const int64_t* out_strides, float scale, int nsplit, void* stream);
 
 /* Cache row mover.
  * Replaces the Tensor.copy_ sequences of HF:306-336 (update_text), HF:340-398

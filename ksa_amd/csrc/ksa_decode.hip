@@ -17,6 +17,8 @@
 #include <hip/hip_runtime.h>
 #include <math.h>
 
+#include <mutex>
+
 #include "ksa_api_internal.h"
 #include "ksa_tile.h"
 
@@ -324,12 +326,13 @@ extern "C" int ksa_decode_auto_splits(int batch, int Hkv, int max_rows) {
     return n < 1 ? 1 : n;
 }
 
-extern "C" int ksa_decode_fwd(const void* q, const void* kcache, const void* vcache, void* out,
-                              const int32_t* start, const int32_t* end, int start0, int end0,
-                              int batch, int Hq, int Hkv, int Q, int D, int dtype,
-                              const int64_t* q_strides, const int64_t* k_strides,
-                              const int64_t* v_strides, const int64_t* out_strides, float scale,
-                              int nsplit, void* workspace, size_t workspace_bytes, void* stream) {
+namespace {
+
+int decode_fwd_impl(const void* q, const void* kcache, const void* vcache, void* out,
+                    const int32_t* start, const int32_t* end, int start0, int end0, int batch, int Hq,
+                    int Hkv, int Q, int D, int dtype, const int64_t* q_strides,
+                    const int64_t* k_strides, const int64_t* v_strides, const int64_t* out_strides,
+                    float scale, int nsplit, void* workspace, size_t workspace_bytes, void* stream) {
     if (!q || !kcache || !vcache || !out || !q_strides || !k_strides || !v_strides || !out_strides)
         return KSA_ERR_NULL;
     if ((start == nullptr) != (end == nullptr)) return KSA_ERR_NULL;
@@ -378,4 +381,71 @@ extern "C" int ksa_decode_fwd(const void* q, const void* kcache, const void* vca
         if (D == 64) return launch<KsaF16, 64>(p, batch, st);
     }
     return KSA_ERR_UNSUPPORTED;
+}
+
+// ---- scratch of the entry point that allocates nothing ----
+// Split-K partials of ksa_decode_fwd_noalloc live in this array instead of a caller-provided
+// workspace.  Every GPU the library is loaded on holds its own copy at its own address; the
+// array's name is only a host-side handle, so the device address is asked for once per device
+// (hipGetSymbolAddress) and kept.
+constexpr size_t kNoAllocScratchBytes = KSA_DECODE_NOALLOC_SCRATCH_BYTES;
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// device address of `scratch` on the current device, or null
+void* noalloc_scratch() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        g_scratch_ptr[dev] = ptr;
+    }
+    return g_scratch_ptr[dev];
+}
+
+}  // namespace
+
+extern "C" int ksa_decode_fwd(const void* q, const void* kcache, const void* vcache, void* out,
+                              const int32_t* start, const int32_t* end, int start0, int end0,
+                              int batch, int Hq, int Hkv, int Q, int D, int dtype,
+                              const int64_t* q_strides, const int64_t* k_strides,
+                              const int64_t* v_strides, const int64_t* out_strides, float scale,
+                              int nsplit, void* workspace, size_t workspace_bytes, void* stream) {
+    return decode_fwd_impl(q, kcache, vcache, out, start, end, start0, end0, batch, Hq, Hkv, Q, D, dtype,
+                           q_strides, k_strides, v_strides, out_strides, scale, nsplit, workspace,
+                           workspace_bytes, stream);
+}
+
+extern "C" size_t ksa_decode_noalloc_max_workspace_bytes(void) { return kNoAllocScratchBytes; }
+
+// ksa_decode_fwd without the workspace arguments: the split-K partials go to the library's own
+// fixed device array.  Nothing is allocated, freed or synchronised here; the kernels are the
+// ones ksa_decode_fwd launches and receive the array's device address as their workspace.
+// Every (sequence, kv head, split, column) slot the merge kernel reads is written by the
+// decode kernel of the same call, so nothing has to be cleared between calls.
+extern "C" int ksa_decode_fwd_noalloc(const void* q, const void* kcache, const void* vcache, void* out,
+                                      const int32_t* start, const int32_t* end, int start0, int end0,
+                                      int batch, int Hq, int Hkv, int Q, int D, int dtype,
+                                      const int64_t* q_strides, const int64_t* k_strides,
+                                      const int64_t* v_strides, const int64_t* out_strides,
+                                      float scale, int nsplit, void* stream) {
+    if (nsplit <= 1)
+        return decode_fwd_impl(q, kcache, vcache, out, start, end, start0, end0, batch, Hq, Hkv, Q, D,
+                               dtype, q_strides, k_strides, v_strides, out_strides, scale, nsplit,
+                               nullptr, 0, stream);
+    if (batch <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || Q <= 0) return KSA_ERR_INVALID;
+    const size_t need = ksa_decode_workspace_bytes(batch, Hq, Hkv, Q, D, nsplit);
+    if (need > kNoAllocScratchBytes) return KSA_ERR_WORKSPACE;
+    void* ws = noalloc_scratch();
+    if (!ws) return KSA_ERR_LAUNCH;
+    return decode_fwd_impl(q, kcache, vcache, out, start, end, start0, end0, batch, Hq, Hkv, Q, D, dtype,
+                           q_strides, k_strides, v_strides, out_strides, scale, nsplit, ws,
+                           kNoAllocScratchBytes, stream);
 }
