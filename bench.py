@@ -7,7 +7,9 @@ Prints ONE JSON line.  A "step" is one prefill forward of a single Summary-Atten
 layer on the 128k configuration (1024 chunks x (128 text + 8 summary) rows, 32 query /
 8 KV heads, head_dim 128, bf16); `value` is its non-empty-block TFLOP/s.  The decode
 attention step over the ring-buffer cache (batch 64, 128k logical context) is timed in a
-second region of the same K/W and reported under "decode".  Inputs are synthetic, seeded,
+second region of the same K/W and reported under "decode"; the two smaller prefill configurations, the fused pre-attention step
+and the end-to-end decoder of config 4 (batch 8, 32k prompt, 256 greedy steps) follow under their
+own keys.  Inputs are synthetic, seeded,
 and resident in HBM before any timed region.  The block index is built once before the
 timed region (the reference caches it the same way); reading the summary prefix is inside.
 """
@@ -107,6 +109,34 @@ def sustained_rate(fn, flop_per_call, seconds, batch):
     return flop_per_call * (n - n_half) / (t - t_half) / 1e12, (sum(late) / len(late) if late else None)
 
 
+def prefill_record(name, chunks, Hq, Hkv, D, C, S, W, dev, steps, warmup, idle):
+    """One prefill configuration timed like the main one: inputs resident, index cached, `steps`
+    launches after `warmup`; returns a record with its own roofline object."""
+    import torch
+    import ksa_amd
+    Sq, P = chunks * (C + S), chunks * S
+    q, k, v, sp = prefill_inputs(chunks, Hq, Hkv, D, C, S, dev, seed=0)
+    idx = ksa_amd.compute_block_sparsity(Sq, Sq + P, C, S, W)
+    tiles = int((idx[0] + idx[2]).sum())
+    flops = 4.0 * 128 * 64 * D * Hq * tiles
+
+    def step():
+        ksa_amd.summary_attn_func(q, k, v, C, S, W, summary_pos=sp)
+
+    torch.cuda.synchronize()
+    time.sleep(idle)
+    wall, dev_ms = time_region(step, steps, warmup)
+    kern_ms = dev_ms / steps
+    return {
+        "workload": name, "chunks": chunks, "seqlen_q": Sq, "q_heads": Hq, "kv_heads": Hkv, "head_dim": D,
+        "sliding_chunk_num": W, "non_empty_tiles_128x64": tiles, "non_empty_block_tflop": flops / 1e12,
+        "steps": steps, "ms_per_step": wall * 1e3 / steps,
+        "roofline": {"bound": "mfma", "achieved": flops / (kern_ms * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "frac": flops / (kern_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+                     "traffic": None, "kernel": "ksa_prefill_kernel<bf16,128>", "kernel_ms": kern_ms},
+    }
+
+
 def cpu_baseline_prefill(chunks, Hq, Hkv, D, C, S, W, tiles_per_mtile, budget_s=20.0):
     """The reference's CPU path (block mode, restated in oracle/cpu_path.py) on a bounded
     sample of 4096-row query blocks; rate in the same non-empty-block TFLOP/s unit."""
@@ -178,15 +208,19 @@ def main():
     ap.add_argument("--skip-pre-attention", action="store_true",
                     help="do not time the fused pre-attention step (q/k RMSNorm + rotary + layout write "
                          "at the prefill shape, reported under 'pre_attention')")
-    ap.add_argument("--sustain", type=float, default=0.0, metavar="SECONDS",
+    ap.add_argument("--sustain", type=float, default=3.0, metavar="SECONDS",
                     help="also loop the prefill launch for SECONDS and report the rate of the second "
-                         "half under 'sustained' (the chip lowers its clock under a long MFMA load)")
-    ap.add_argument("--e2e", action="store_true",
-                    help="also run the end-to-end decoder (random-init 4B shape: 36 layers, 3 Summary : 1 "
-                         "full, batch 8, 32k-token prompt, 256 greedy steps) and report prefill and "
-                         "decode tokens/s under 'e2e'")
-    ap.add_argument("--e2e-graph", action="store_true",
-                    help="replay the non-boundary decode steps of --e2e from a HIP graph")
+                         "half under 'sustained' (the chip lowers its clock under a long MFMA load); 0 = skip")
+    ap.add_argument("--skip-small-prefill", action="store_true",
+                    help="do not time the two smaller prefill configurations (cfg 0: 32 chunks, 16/8 heads; "
+                         "cfg 1: 256 chunks, 32/8 heads), reported under 'prefill_cfg0' / 'prefill_cfg1'")
+    ap.add_argument("--no-e2e", action="store_true",
+                    help="skip the end-to-end decoder (random-init 4B shape: 36 layers, 3 Summary : 1 "
+                         "full, batch 8, 32k-token prompt, 256 greedy steps; prefill and decode tokens/s "
+                         "under 'e2e')")
+    ap.add_argument("--e2e-eager", action="store_true",
+                    help="launch the decode steps of the end-to-end run one kernel at a time instead of "
+                         "replaying the non-boundary steps from a HIP graph")
     ap.add_argument("--e2e-batch", type=int, default=8)
     ap.add_argument("--e2e-prompt", type=int, default=32768)
     ap.add_argument("--e2e-new", type=int, default=256)
@@ -195,6 +229,8 @@ def main():
                     help="also run one ksa_copy_rows of 1 GiB (a plain copy kernel of known size, "
                          "used to scale the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     args = ap.parse_args()
+    args.e2e = not args.no_e2e
+    args.e2e_graph = not args.e2e_eager
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (both kernels shard "
               "by head / sequence with no communication); run with --gpus 1", file=sys.stderr)
@@ -271,6 +307,13 @@ def main():
                                    "frac_of_peak": rate / PEAK_BF16_TFLOPS, "sclk_mhz_mean": clk}
         del q, k, v, sp
         torch.cuda.empty_cache()
+        if not args.skip_small_prefill and chunks == 1024:
+            # the two smaller configurations of the same kernel (launches of 30 us and 1 ms:
+            # more of them per region)
+            result["prefill_cfg0"] = prefill_record("cfg0-prefill-32-chunks-16q8kv", 32, 16, 8, D, C, S, W, dev,
+                                                    args.steps * 20, args.warmup * 4, args.idle)
+            result["prefill_cfg1"] = prefill_record("cfg1-prefill-32k", 256, Hq, Hkv, D, C, S, W, dev,
+                                                    args.steps * 4, args.warmup * 2, args.idle)
 
     # ------------------------------------------------------------------ decode
     if not args.skip_decode:
@@ -353,7 +396,7 @@ def main():
         del qkv, qo, ko, vo, cosb, sinb, emb, ang
         torch.cuda.empty_cache()
 
-    # ------------------------------------------------------------------ CPU baseline
+    # ------------------------------------------------------------------ end-to-end decoder (config 4)
     if args.e2e:
         from ksa_amd.model import KsaQwen3Config, KsaQwen3ForCausalLM, init_weights
         nl = args.e2e_layers
@@ -369,6 +412,15 @@ def main():
         logits, cache = model.prefill(ids)
         torch.cuda.synchronize()
         t_prefill = time.perf_counter() - t0
+
+        def attended_rows():   # cache rows one decode step reads, summed over the layers
+            return sum(e - a for a, e in (cache.attention_range(li) for li in range(nl)))
+
+        def matrix_bytes():    # weights one decode step reads: every layer's matrices and the output head
+            n = sum(w.numel() for lw in weights["layers"] for w in lw.values())
+            return (n + model.lm_head.numel() + weights["norm"].numel()) * 2
+
+        rows_first = attended_rows()
         t0 = time.perf_counter()
         n_boundary = 0
         for _ in range(args.e2e_new):
@@ -377,6 +429,9 @@ def main():
             logits = model.decode_step_graph(nxt, cache) if args.e2e_graph else model.decode_step(nxt, cache)
         torch.cuda.synchronize()
         t_decode = time.perf_counter() - t0
+        rows_mean = (rows_first + attended_rows()) / 2
+        step_bytes = matrix_bytes() + 2 * rows_mean * cfg.num_key_value_heads * cfg.head_dim * 2 * args.e2e_batch
+        floor_ms = step_bytes / (PEAK_HBM_GBPS * 1e9) * 1e3
         result["e2e"] = {
             "workload": f"random-init decoder, {nl} layers (3 Summary W={W} : 1 unbounded window), hidden "
                         f"{cfg.hidden_size}, {Hq}/{Hkv} heads, batch {args.e2e_batch}, prompt "
@@ -385,6 +440,8 @@ def main():
             "decode_s": t_decode, "decode_ms_per_step": t_decode / args.e2e_new * 1e3,
             "decode_tokens_per_s": args.e2e_batch * args.e2e_new / t_decode,
             "chunk_boundary_steps": int(n_boundary), "decode_hip_graph": bool(args.e2e_graph),
+            "decode_step_bytes": int(step_bytes), "decode_hbm_floor_ms": floor_ms,
+            "decode_frac_of_hbm_floor": floor_ms / (t_decode / args.e2e_new * 1e3),
             "hbm_allocated_gb": torch.cuda.max_memory_allocated() / 1e9,
         }
         del model, weights, cache, logits
