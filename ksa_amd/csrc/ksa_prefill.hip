@@ -685,17 +685,29 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
             constexpr float kMinRowSum = std::is_same<T, KsaF16>::value ? 0.0625f : 5.4e-20f;
             bad = bad || !(l_tot > kMinRowSum);
         }
-        if (__syncthreads_or(bad)) walk(std::true_type{});
+        if (__syncthreads_or(bad)) {
+            walk(std::true_type{});
+            __syncthreads();  // the epilogue reuses the tiles' LDS
+        }
     }
 
     // ---- epilogue ----
+    // The normalised rows go to global memory through LDS (the K/V tiles are dead by now): in the
+    // accumulator layout a lane holds 4-element pieces of its query row, and a store instruction
+    // straight from there would touch 32 rows in 16-byte pieces; turned around in LDS, every
+    // store instruction writes four whole rows of 2 D bytes (3 us less per workgroup).  A wave's
+    // 32-row block has its own LDS region (16-byte chunk c of row r at position c ^ (r % CPR):
+    // conflict-free both ways), so waves do not wait for each other.
     if constexpr (RB != 1) ksa_mfma_settle();
+    {
+        const int q0 = wave_u * RB;  // first region of this wave; two regions per 64-row LDS array
 #pragma unroll
-    for (int r = 0; r < RB; ++r) {
-        const float l_tot = ksa_pair_sum(l_run[r]);
-        const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-        if (qrow[r] < mk.Sq) {
-            uint16_t* op = p.out + bz * p.o_bs + (int64_t)qrow[r] * p.o_rs + head * p.o_hs;
+        for (int r = 0; r < RB; ++r) {
+            const float l_tot = ksa_pair_sum(l_run[r]);
+            const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+            const int qreg = q0 + r;
+            uint16_t* arr = (qreg >> 1) == 0 ? Ks0 : (qreg >> 1) == 1 ? Ks1 : (qreg >> 1) == 2 ? Vs0 : Vs1;
+            char* region = reinterpret_cast<char*>(arr) + (qreg & 1) * 32 * ROWB;
 #pragma unroll
             for (int b = 0; b < DB; ++b)
 #pragma unroll
@@ -703,9 +715,21 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
                     u32x2 w;
                     w[0] = Ops::pack2(oacc[r][b][4 * j] * inv, oacc[r][b][4 * j + 1] * inv);
                     w[1] = Ops::pack2(oacc[r][b][4 * j + 2] * inv, oacc[r][b][4 * j + 3] * inv);
-                    *reinterpret_cast<u32x2*>(op + 32 * b + 8 * j + 4 * lh) = w;
+                    const int pch = (4 * b + j) ^ (lq & (CPR - 1));
+                    *reinterpret_cast<u32x2*>(region + lq * ROWB + pch * 16 + 8 * lh) = w;
                 }
-            if (p.lse && lh == 0)
+            ksa_wave_lds_fence();
+            const int brow0 = row0 + 32 * r;  // first query row of the block
+            uint16_t* ob = p.out + bz * p.o_bs + head * p.o_hs;
+#pragma unroll
+            for (int i = 0; i < (32 * CPR) / 64; ++i) {
+                const int idx = i * 64 + lane;
+                const int row = idx / CPR, c = idx % CPR;
+                const u32x4 w = *reinterpret_cast<const u32x4*>(region + row * ROWB + ((c ^ (row & (CPR - 1))) * 16));
+                if (brow0 + row < mk.Sq)
+                    *reinterpret_cast<u32x4*>(ob + (int64_t)(brow0 + row) * p.o_rs + 8 * c) = w;
+            }
+            if (p.lse && lh == 0 && qrow[r] < mk.Sq)
                 p.lse[bz * p.lse_bs + head * p.lse_hs + qrow[r]] =
                     l_tot > 0.f ? m_ref[r] * p.scale + logf(l_tot) : -INFINITY;
         }
