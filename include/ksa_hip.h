@@ -72,7 +72,13 @@ int ksa_block_index(int Sq, int Sk, int C, int S, int W, int P, int skip_old, in
  *   shape: workgroup shape, a tuning knob with no effect on the result beyond the tolerance of
  *       the tests.  KSA_PREFILL_SHAPE_AUTO lets the library choose from the launch size and the
  *       device's CU count; the others apply to head_dim 128 with an even Hq / Hkv and fall back
- *       to one head per workgroup elsewhere. */
+ *       to one head per workgroup elsewhere.
+ *   sched: NULL, or 8 int32 of device memory for this call alone (contents irrelevant on entry,
+ *       undefined afterwards; calls that may overlap in time need one each).  With it, a long
+ *       launch hands out its last, light work items from per-XCD queues (device-scope atomics)
+ *       instead of a fixed split, so that XCDs running at slightly different clocks end together;
+ *       one small extra kernel in front of the launch clears the counters.  No effect on the
+ *       result. */
 #define KSA_PREFILL_SHAPE_AUTO 0       /* library's choice */
 #define KSA_PREFILL_SHAPE_1HEAD 32     /* one query head on 4 waves, 32 rows per wave */
 #define KSA_PREFILL_SHAPE_2HEAD_64 64  /* two heads of a kv group on 4 waves, 64 rows per wave */
@@ -82,7 +88,7 @@ int ksa_prefill_fwd(const void* q, const void* k, const void* v, void* out, floa
                     const int64_t* kv_strides, const int64_t* out_strides, int C, int S, int W,
                     int P, int skip_old, int phys_prefix, const int32_t* mask_cnt,
                     const int32_t* mask_idx, const int32_t* full_cnt, const int32_t* full_idx,
-                    int idx_stride, float scale, int shape, void* stream);
+                    int idx_stride, float scale, int shape, int32_t* sched, void* stream);
 
 /* Decode attention over the ring-buffer slice.
  * Replaces HF:591-612 (_sdpa_attention_forward, incl. repeat_kv :557-566) applied to the

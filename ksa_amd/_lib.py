@@ -23,7 +23,7 @@ _SIGNATURES = {
     "ksa_device_cu_count": (_int, []),
     "ksa_block_index": (_int, [_int] * 9 + [_vp] * 4 + [_vp]),
     "ksa_prefill_fwd": (_int, [_vp] * 5 + [_int] * 6 + [_i64p] * 3 + [_int] * 6 + [_vp] * 4
-                        + [_int, ctypes.c_float, _int, _vp]),
+                        + [_int, ctypes.c_float, _int, _vp, _vp]),
     "ksa_decode_workspace_bytes": (ctypes.c_size_t, [_int] * 6),
     "ksa_decode_auto_splits": (_int, [_int] * 3),
     "ksa_decode_fwd": (_int, [_vp] * 6 + [_int] * 8 + [_i64p] * 4

@@ -66,6 +66,18 @@ struct PrefillParams {
     float scale;
     float scale_log2;
     int shape;  // 2: two heads on 8 waves; 32: one head per workgroup; 64: two heads, 64 query rows per wave
+    // Work items (batch element, m tile, head (pair), kv head) are numbered heavy first; workgroup
+    // i takes item i while i < n_static.  The workgroups behind that take the remaining (light)
+    // items from eight queues in device memory, one per XCD (queue = item number modulo 8, which is
+    // also the XCD a workgroup of that number runs on and the kv head whose K/V that XCD's cache
+    // holds): first from the queue of their own XCD, then from the others.  The XCDs of one chip
+    // run at clocks a few per cent apart; with a fixed split the launch ends when the slowest one
+    // is done, with the queues the faster ones take over part of its tail.  sched == null: all
+    // workgroups take the item of their own number.
+    int32_t* sched;   // eight counters, zeroed in front of the launch
+    int n_items;      // items per batch element
+    int total;        // items in all
+    int n_static;     // multiple of 8
 };
 
 constexpr int kTileM = 128;
@@ -158,8 +170,24 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
 
     // workgroup -> (kv head, query head (pair) in group, m tile); kv head fastest so that
     // the workgroups sharing K/V land on one XCD; heavy (late) m tiles first.
-    const int bz = blockIdx.y;
-    const int id = blockIdx.x;
+    int item = blockIdx.x;
+    if (p.sched != nullptr && item >= p.n_static) {
+        __shared__ int s_item;
+        if (tid == 0) {
+            int got = -1;
+            for (int k = 0; k < 8 && got < 0; ++k) {
+                const int y = (item + k) & 7;
+                const int cand = p.n_static + y + 8 * atomicAdd(&p.sched[y], 1);
+                if (cand < p.total) got = cand;
+            }
+            s_item = got;
+        }
+        __syncthreads();
+        item = s_item;
+        if (item < 0) return;  // every queue is empty: a spare workgroup
+    }
+    const int bz = item / p.n_items;
+    const int id = item - bz * p.n_items;
     const int kvh = id % p.Hkv;
     const int rest = id / p.Hkv;
     constexpr int kWavesPerHead = 4 / RB;
@@ -736,6 +764,10 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
     }
 }
 
+__global__ void ksa_prefill_zero_queues_kernel(int32_t* sched) {
+    if (threadIdx.x < 8) sched[threadIdx.x] = 0;
+}
+
 template <typename T, int D, int RB, int HW>
 int launch_shape(const PrefillParams& p, int batch, hipStream_t stream) {
     constexpr int kThreads = PrefillShape<RB, HW>::kThreads;
@@ -743,11 +775,27 @@ int launch_shape(const PrefillParams& p, int batch, hipStream_t stream) {
     const KsaMask& mk = p.mk;
     const bool prefix_ok = mk.P == 0 || p.phys_prefix || (RSTEP % mk.S == 0 && mk.P % kTileN == 0);
     const bool regular = prefix_ok && mk.Sk % kTileN == 0;
-    dim3 grid(p.M * (p.Hq / HW), batch);
+    PrefillParams pp = p;
+    pp.n_items = p.M * (p.Hq / HW);
+    pp.total = pp.n_items * batch;
+    pp.n_static = pp.total;
+    int spare = 0;
+    // Queues only for long launches (32 workgroups per CU and more; measured at 128k rows: +2.2 %,
+    // at 32k rows with 17 per CU: -0.8 %), where the tail they even out is worth the clearing kernel
+    // and the atomic in front of the light items: the last 30 % of the items, with a quarter more
+    // workgroups than items there (the spare ones find the queues empty and leave).
+    if (p.sched != nullptr && (int64_t)pp.total >= 32ll * ksa_cu_count_or(256)) {
+        pp.n_static = (int)((int64_t)pp.total * 7 / 10) / 8 * 8;
+        spare = ((pp.total - pp.n_static) / 4 + 7) / 8 * 8;
+        hipLaunchKernelGGL(ksa_prefill_zero_queues_kernel, dim3(1), dim3(64), 0, stream, p.sched);
+    } else {
+        pp.sched = nullptr;
+    }
+    dim3 grid(pp.total + spare);
     if (regular)
-        hipLaunchKernelGGL((ksa_prefill_kernel<T, D, true, RB, HW>), grid, dim3(kThreads), 0, stream, p);
+        hipLaunchKernelGGL((ksa_prefill_kernel<T, D, true, RB, HW>), grid, dim3(kThreads), 0, stream, pp);
     else
-        hipLaunchKernelGGL((ksa_prefill_kernel<T, D, false, RB, HW>), grid, dim3(kThreads), 0, stream, p);
+        hipLaunchKernelGGL((ksa_prefill_kernel<T, D, false, RB, HW>), grid, dim3(kThreads), 0, stream, pp);
     return ksa_check_launch();
 }
 
@@ -775,7 +823,7 @@ extern "C" int ksa_prefill_fwd(const void* q, const void* k, const void* v, void
                                int skip_old, int phys_prefix, const int32_t* mask_cnt,
                                const int32_t* mask_idx, const int32_t* full_cnt,
                                const int32_t* full_idx, int idx_stride, float scale, int shape,
-                               void* stream) {
+                               int32_t* sched, void* stream) {
     if (!q || !k || !v || !out || !mask_cnt || !mask_idx || !full_cnt || !full_idx) return KSA_ERR_NULL;
     if (!q_strides || !kv_strides || !out_strides) return KSA_ERR_NULL;
     if (batch <= 0 || Sq <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0) return KSA_ERR_INVALID;
@@ -823,6 +871,7 @@ extern "C" int ksa_prefill_fwd(const void* q, const void* k, const void* v, void
     p.mk = KsaMask{C, S, W, P, skip_old ? 1 : 0, Sq, Sk};
     p.scale = scale;
     p.scale_log2 = scale * 1.4426950408889634f;
+    p.sched = sched;
     // Workgroup shape (D = 128, even group size; anything else uses one head per workgroup):
     // 2 = two heads on 8 waves; 32 = one head on 4 waves; 64 = two heads on 4 waves with 64 query
     // rows per wave (one wave per SIMD).  Left to the library (0), a short launch (fewer than 16

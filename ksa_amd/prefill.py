@@ -160,6 +160,7 @@ def _summary_attn_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     Hkv = k.shape[2]
     out = torch.empty_like(q)
     lse = torch.empty((b, Hq, Sq) if want_lse else (0,), dtype=torch.float32, device=q.device)
+    sched = torch.empty(8, dtype=torch.int32, device=q.device)   # work queues of this call alone
     dims = (0, 1, 2)
     with torch.cuda.device(q.device):
         rc = _lib.lib().ksa_prefill_fwd(
@@ -169,7 +170,7 @@ def _summary_attn_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
             _lib.strides3(q, dims), _lib.strides3(k, dims), _lib.strides3(out, dims),
             C, S, W, P, int(skip_old), int(phys_prefix),
             mask_cnt.data_ptr(), mask_idx.data_ptr(), full_cnt.data_ptr(), full_idx.data_ptr(),
-            mask_idx.shape[-1], float(scale), int(shape), _lib.stream_ptr(q.device))
+            mask_idx.shape[-1], float(scale), int(shape), sched.data_ptr(), _lib.stream_ptr(q.device))
     _lib.check(rc, "ksa_prefill_fwd")
     return out, lse
 

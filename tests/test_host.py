@@ -40,7 +40,7 @@ def test_error_codes_before_launch():
     assert L.ksa_block_index(100, 110, 128, 8, 3, 10, 0, 128, 64, None, None, None, None, None) == -2
     null3 = ctypes.cast(None, ctypes.POINTER(ctypes.c_int64))
     assert L.ksa_prefill_fwd(None, None, None, None, None, 1, 128, 4, 2, 128, 0, null3, null3, null3,
-                             128, 8, 3, 0, 0, 0, None, None, None, None, 2, 1.0, 0, None) == -2
+                             128, 8, 3, 0, 0, 0, None, None, None, None, 2, 1.0, 0, None, None) == -2
     assert L.ksa_decode_fwd(None, None, None, None, None, None, 0, 10, 1, 4, 2, 1, 128, 0, null3, null3,
                             null3, null3, 1.0, 1, None, 0, None) == -2
     assert L.ksa_decode_workspace_bytes(64, 32, 8, 1, 128, 1) == 0

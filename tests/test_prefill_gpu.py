@@ -261,6 +261,29 @@ def test_prefill_cfg2_sampled_rows():
     assert np.abs(lse[:, rows] - wlse).max() <= 2e-3
 
 
+def test_prefill_work_queues_equal_fixed_split():
+    """A long launch (32 workgroups per CU and more) hands out its last work items from per-XCD
+    queues; a short one gives workgroup i item i.  Three copies of a 32k-row sequence in one batch
+    take the first path, one copy the second: every copy must equal it bit for bit (an item
+    skipped or computed for the wrong batch element would show), with and without the queues'
+    memory, on two launches in a row."""
+    import ksa_amd
+    from ksa_amd import _lib
+    dev = torch.device("cuda")
+    Sq, Hq, Hkv, D, C, S, W = 34816, 32, 8, 128, 128, 8, 4
+    q, k, v = make_qkv(Sq, Hq, Hkv, D, seed=21)
+    sp = torch.as_tensor(O.summary_positions(Sq, C, S), device=dev)
+    q1, k1, v1 = q[None].to(dev), k[None].to(dev), v[None].to(dev)
+    one, _ = ksa_amd.summary_attn_func(q1, k1, v1, C, S, W, summary_pos=sp)
+    assert Sq // 128 * (Hq // 2) < 32 * _lib.lib().ksa_device_cu_count() <= 3 * (Sq // 128) * (Hq // 2)
+    q3, k3, v3 = (t.expand(3, -1, -1, -1).contiguous() for t in (q1, k1, v1))
+    for _ in range(2):
+        three, _ = ksa_amd.summary_attn_func(q3, k3, v3, C, S, W, summary_pos=sp)
+        torch.cuda.synchronize()
+        for b in range(3):
+            assert torch.equal(three[b], one[0]), b
+
+
 def test_prefill_cfg2_visibility_probe_all_rows():
     """Every row of the 128k shape: with Q = K = 0 and V = one-hot of (position mod 128) the
     output is count-of-class / n_i over the row's visible set.  All probabilities are exactly 1,
