@@ -471,6 +471,9 @@ def main():
                 result["decode"]["roofline"]["traffic"] = t.get("decode_bytes_per_launch")
             if "pre_attention" in result and t.get("pre_attention_workload") == result["pre_attention"]["workload"]:
                 result["pre_attention"]["roofline"]["traffic"] = t.get("pre_attention_bytes_per_launch")
+            for key in ("prefill_cfg0", "prefill_cfg1"):
+                if key in result and result[key]["workload"] == t.get(key + "_workload"):
+                    result[key]["roofline"]["traffic"] = t.get(key + "_bytes_per_launch")
         except Exception:
             pass
     print(json.dumps(result))
