@@ -122,7 +122,10 @@ __global__ __launch_bounds__(256) void ksa_pre_attention_kernel(const PreParams 
     // it works on the current one, so two of its row requests are in flight.
     const int TOK = p.tok_per_pass;
     const int span = p.passes_per_wg * TOK;  // consecutive tokens of one workgroup
-    int gi = wave % G, tl = wave / G, t0 = blockIdx.x * span;
+    // (a handful of tokens: gridDim.y workgroups share a token, each taking every gridDim.y-th set
+    // of four row groups, so that no wave has more than one group to do)
+    const int gstep = 4 * gridDim.y;
+    int gi = (wave + 4 * blockIdx.y) % G, tl = (wave + 4 * blockIdx.y) / G, t0 = blockIdx.x * span;
     const int t_end = min(ntok, t0 + span);
     struct Group {
         bool live;             // wave-uniform: there is such a group
@@ -156,7 +159,7 @@ __global__ __launch_bounds__(256) void ksa_pre_attention_kernel(const PreParams 
         // (k and v may go to a row of their sequence that the host does not know: a cache cursor)
         const int64_t drow = ns + ((g.which != 0 && p.kv_row) ? p.kv_row[nb] : 0);
         g.dbase = p.dst[g.which] + nb * p.d_bs[g.which] + drow * p.d_rs[g.which] + (int64_t)g.h0 * p.d_hs[g.which];
-        gi += 4;
+        gi += gstep;
         return g;
     };
     auto pick = [](int which, const uint32_t (&a)[3]) { return which == 0 ? a[0] : (which == 1 ? a[1] : a[2]); };
@@ -259,10 +262,14 @@ int launch_pre(PreParams p, hipStream_t stream) {
     p.passes_per_wg = (int64_t)p.batch * p.S / p.tok_per_pass >= 4 * 1024 ? 4 : 1;
     const int64_t span = (int64_t)p.passes_per_wg * p.tok_per_pass;
     const int64_t blocks = ((int64_t)p.batch * p.S + span - 1) / span;
+    // a decode step (one pass of one token per workgroup): one workgroup per four row groups of a
+    // token instead of one per token - the groups of a wave are a chain of dependent loads
+    const int parts = (p.passes_per_wg == 1 && p.tok_per_pass == 1 && blocks <= 64) ? G / 4 : 1;
+    const dim3 grid((unsigned)blocks, (unsigned)parts);
     if (p.part)
-        hipLaunchKernelGGL((ksa_pre_attention_kernel<T, D, true>), dim3((unsigned)blocks), dim3(256), 0, stream, p);
+        hipLaunchKernelGGL((ksa_pre_attention_kernel<T, D, true>), grid, dim3(256), 0, stream, p);
     else
-        hipLaunchKernelGGL((ksa_pre_attention_kernel<T, D, false>), dim3((unsigned)blocks), dim3(256), 0, stream, p);
+        hipLaunchKernelGGL((ksa_pre_attention_kernel<T, D, false>), grid, dim3(256), 0, stream, p);
     return ksa_check_launch();
 }
 
