@@ -142,3 +142,27 @@ def test_copy_rows():
     idx = torch.tensor([7, 3, 49, 0], dtype=torch.int32, device=dev)
     _move_rows(src, dst, 4, dst_start=60, src_index=idx)
     assert torch.equal(dst[:, :, 60:64], src[:, :, idx.long()])
+
+
+def test_decode_empty_and_single_row_ranges():
+    """Ragged extremes: a sequence whose row range is empty (the reference never produces one; this
+    build defines its output as zeros, not NaN), one with a single row (output = that row of V) and
+    ordinary ones in the same launch, with one and with several splits."""
+    import ksa_amd
+    dev = torch.device("cuda")
+    g = torch.Generator().manual_seed(31)
+    b, Hq, Hkv, D, rows = 4, 8, 2, 128, 900
+    q = torch.randn(b, Hq, 1, D, generator=g).bfloat16()
+    kc = torch.randn(b, Hkv, rows, D, generator=g).bfloat16()
+    vc = torch.randn(b, Hkv, rows, D, generator=g).bfloat16()
+    start = np.array([100, 500, 0, 37], np.int32)
+    end = np.array([100, 501, 900, 300], np.int32)
+    for nsplit in (1, 4):
+        got = ksa_amd.ksa_decode(q.to(dev), kc.to(dev), vc.to(dev), torch.as_tensor(start, device=dev),
+                                 torch.as_tensor(end, device=dev), nsplit=nsplit).float().cpu().numpy()
+        assert np.isfinite(got).all()
+        assert np.abs(got[0]).max() == 0.0
+        want1 = vc[1, :, 500].float().numpy()                     # [Hkv, D]; head h reads kv head h // g
+        assert np.array_equal(got[1, 0], np.repeat(want1, Hq // Hkv, axis=0))
+        ref = c_oracle.decode(q[2:].float().numpy(), kc[2:].float().numpy(), vc[2:].float().numpy(), start[2:], end[2:])
+        assert np.abs(got[2:] - ref).max() <= 2e-2
