@@ -225,6 +225,19 @@ int ksa_gemm_rows(const void* x, const void* w, void* out, int M, int N, int K, 
                   long long w_row_stride, long long out_row_stride, int dtype, int ksplit,
                   void* workspace, size_t workspace_bytes, void* stream);
 
+/* The MLP's gate | up projection with its activation folded in, for at most 16 rows of x:
+ * out = round(SiLU(round(x w_gate^T))) * round(x w_up^T), one launch, no partial sums in memory.
+ * Replaces act_fn(gate_proj(x)) * up_proj(x) of Qwen3MLP.forward (HF:507-514) at a decode step, i.e.
+ * ksa_gemm_rows on the fused gate | up matrix followed by ksa_silu_mul (same rounding points; the
+ * fp32 sums run over K in one chain instead of split-K order, so the 16-bit results can differ from
+ * that pair's in the last place).
+ *   x [M, K], w [2 I, K] (gate rows, then up rows), out [M, I]; K a multiple of 32; row strides in
+ *   elements (x, w: multiples of 8).  x is held in LDS whole: M (K + 8) 2 bytes beyond 160 KiB are
+ *   KSA_ERR_UNSUPPORTED (use ksa_gemm_rows and ksa_silu_mul then). */
+int ksa_gemm_rows_gate_up_silu(const void* x, const void* w, void* out, int M, int I, int K,
+                               long long x_row_stride, long long w_row_stride, long long out_row_stride,
+                               int dtype, void* stream);
+
 /* Host-side diagnostic: number of key columns in [a, b) visible to query row q under the
  * closed-form rule the kernels use (no GPU involved). */
 long long ksa_debug_count_visible(long long q, long long a, long long b, int C, int S, int W,

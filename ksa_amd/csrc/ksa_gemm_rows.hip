@@ -131,6 +131,99 @@ int launch_gemm(const GemmParams& p, hipStream_t st) {
     return ksa_check_launch();
 }
 
+// ---- gate | up projection with the MLP's activation folded in ----
+// out[m][n] = round(SiLU(round(x . w[n]))) * round(x . w[I + n]) for the few rows of a decode step
+// (examples/pretrain/hf_template/modeling_qwen3sa.py:507-514, act_fn(gate_proj(x)) * up_proj(x), with
+// the rounding points of its 16-bit tensor ops).  A workgroup owns 16 columns of the hidden vector
+// and the whole of K: wave (h, s) multiplies the chunks s, s + S, ... of 512 elements of K with the
+// gate (h = 0) or up (h = 1) rows of w, where S = min(chunks of K, 8) - at K = 2560 ten waves with
+// one chunk each and no loop, every weight load of the workgroup in flight at once.  x is staged in
+// LDS once, whole; the partial sums of the 2 S waves meet in LDS (in place of x), and the first 256
+// threads finish one output each.  Product, activation and multiply are one launch and no partial
+// sums travel through memory.
+struct GateUpParams {
+    const uint16_t* x;   // [M, K]
+    const uint16_t* w;   // [2 I, K]: gate rows, then up rows
+    uint16_t* out;       // [M, I]
+    int64_t xs, ws, os;
+    int M, I, K, S;      // S: K slices = waves per half
+};
+constexpr int kGateUpMaxSlices = 8;
+
+static inline size_t gate_up_lds_bytes(int M, int K, int S) {
+    const size_t xb = (size_t)M * (K + 8) * 2;
+    const size_t rb = (size_t)2 * S * 16 * 17 * sizeof(float);
+    return xb > rb ? xb : rb;
+}
+
+template <typename T>
+__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) void ksa_gemm_gate_up_silu_kernel(const GateUpParams p) {
+    using C = KsaCvt<T>;
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int r = lane & 15;
+    const int kq = lane >> 4;
+    const int half = wave / p.S;  // 0: gate rows of w, 1: up rows
+    const int slice = wave - half * p.S;
+    const int n0 = blockIdx.x * 16;
+    const int steps = p.K / 32;
+    const int chunks = (steps + kChunkSteps - 1) / kChunkSteps;
+    const int rowb = (p.K + 8) * 2;
+    const uint16_t* wp = p.w + ((int64_t)half * p.I + min(n0 + r, p.I - 1)) * p.ws + 8 * kq;
+    const int xrow = min(r, p.M - 1);
+
+    // eight K steps of weights in flight per wave (32 registers): with at most 64 registers a SIMD
+    // holds eight waves, so three workgroups of ten waves per CU and the whole grid of a 4B-shape
+    // MLP (608 workgroups) is resident at once
+    constexpr int kB = 8;
+    u32x4 a[kB];
+    auto load_steps = [&](int s0) {
+#pragma unroll
+        for (int u = 0; u < kB; ++u) a[u] = *reinterpret_cast<const u32x4*>(wp + 32 * min(s0 + u, steps - 1));
+    };
+    load_steps(slice * kChunkSteps);  // in flight while x is staged (every slice has a first chunk: S <= chunks)
+    const int per_row = p.K / 8;
+    for (int e = threadIdx.x; e < p.M * per_row; e += blockDim.x) {
+        const int m = e / per_row, j = e - m * per_row;
+        *reinterpret_cast<u32x4*>(lds + m * rowb + 16 * j) =
+            *reinterpret_cast<const u32x4*>(p.x + (int64_t)m * p.xs + 8 * j);
+    }
+    __syncthreads();
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int c = slice; c < chunks; c += p.S) {
+        for (int s0 = c * kChunkSteps; s0 < min((c + 1) * kChunkSteps, steps); s0 += kB) {
+            if (s0 != slice * kChunkSteps) load_steps(s0);
+            const int nst = min(kB, steps - s0);
+            const unsigned char* xb = lds + xrow * rowb + s0 * 64 + 16 * kq;
+#pragma unroll
+            for (int u = 0; u < kB; ++u) {
+                if (u < nst) acc = mfma16<T>(a[u], *reinterpret_cast<const u32x4*>(xb + 64 * u), acc);
+            }
+        }
+    }
+    __syncthreads();  // x is no longer read: its place takes the partial sums
+    // C layout of the 16x16 tile: lane holds row of x lane % 16, columns 4 * (lane / 16) + i
+    float* red = reinterpret_cast<float*>(lds);  // [2 S][16 rows][17]
+#pragma unroll
+    for (int i = 0; i < 4; ++i) red[(wave * 16 + r) * 17 + 4 * kq + i] = acc[i];
+    __syncthreads();
+    if (threadIdx.x < 256) {
+        const int m = threadIdx.x >> 4, n = n0 + (threadIdx.x & 15);
+        if (m < p.M && n < p.I) {
+            float g = 0.f, u = 0.f;
+            for (int sl = 0; sl < p.S; ++sl) {
+                g += red[(sl * 16 + m) * 17 + (threadIdx.x & 15)];
+                u += red[((p.S + sl) * 16 + m) * 17 + (threadIdx.x & 15)];
+            }
+            g = C::up(C::down(g));
+            u = C::up(C::down(u));
+            const float act = C::up(C::down(g / (1.f + expf(-g))));
+            p.out[(int64_t)m * p.os + n] = C::down(act * u);
+        }
+    }
+}
+
 }  // namespace
 
 // K splits that give about two workgroups per CU of the current device (256 CUs assumed when no
@@ -176,4 +269,33 @@ extern "C" int ksa_gemm_rows(const void* x, const void* w, void* out, int M, int
     }
     return dtype == KSA_DTYPE_BF16 ? launch_gemm<KsaBf16>(p, (hipStream_t)stream)
                                    : launch_gemm<KsaF16>(p, (hipStream_t)stream);
+}
+
+extern "C" int ksa_gemm_rows_gate_up_silu(const void* x, const void* w, void* out, int M, int I, int K,
+                                          long long x_row_stride, long long w_row_stride,
+                                          long long out_row_stride, int dtype, void* stream) {
+    if (!x || !w || !out) return KSA_ERR_NULL;
+    if (M <= 0 || M > 16 || I <= 0 || K <= 0 || K % 32 != 0) return KSA_ERR_INVALID;
+    if (dtype != KSA_DTYPE_BF16 && dtype != KSA_DTYPE_F16) return KSA_ERR_UNSUPPORTED;
+    if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w)) & 15) return KSA_ERR_ALIGN;
+    if (x_row_stride % 8 || w_row_stride % 8) return KSA_ERR_ALIGN;
+    GateUpParams p{};
+    p.x = (const uint16_t*)x;
+    p.w = (const uint16_t*)w;
+    p.out = (uint16_t*)out;
+    p.xs = x_row_stride, p.ws = w_row_stride, p.os = out_row_stride;
+    p.M = M, p.I = I, p.K = K;
+    const int chunks = (K / 32 + kChunkSteps - 1) / kChunkSteps;
+    p.S = chunks < kGateUpMaxSlices ? chunks : kGateUpMaxSlices;
+    const size_t lds = gate_up_lds_bytes(M, K, p.S);
+    if (lds > 160 * 1024) return KSA_ERR_UNSUPPORTED;  // x does not fit LDS whole: M (K + 8) 2 bytes
+    const dim3 grid((I + 15) / 16), block(128 * p.S);
+    auto kern = dtype == KSA_DTYPE_BF16 ? ksa_gemm_gate_up_silu_kernel<KsaBf16> : ksa_gemm_gate_up_silu_kernel<KsaF16>;
+    if (lds > 64 * 1024) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return KSA_ERR_LAUNCH;
+    }
+    hipLaunchKernelGGL(kern, grid, block, lds, (hipStream_t)stream, p);
+    return ksa_check_launch();
 }

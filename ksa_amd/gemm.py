@@ -57,3 +57,25 @@ def linear_rows(x: torch.Tensor, weight: torch.Tensor, defer: bool = False):
     if defer:
         return SplitKPartials(ws, ks, M, (*x.shape[:-1], N), x.dtype)
     return out.view(*x.shape[:-1], N)
+
+
+def gate_up_silu_rows(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """x [..., K] with at most 16 rows in all, weight [2 I, K] (gate rows, then up rows) ->
+    SiLU(x W_gate^T) * (x W_up^T) [..., I] in one launch (`ksa_gemm_rows_gate_up_silu`): the MLP's
+    `act_fn(gate_proj(x)) * up_proj(x)` (modeling_qwen3sa.py:507-514) at a decode step."""
+    assert x.is_cuda and x.dtype in _DT and weight.dtype == x.dtype, "bf16/fp16 GPU tensors"
+    K = x.shape[-1]
+    I = weight.shape[0] // 2
+    assert weight.shape == (2 * I, K) and weight.stride(1) == 1
+    x2 = x.reshape(-1, K)
+    if x2.stride(1) != 1:
+        x2 = x2.contiguous()
+    M = x2.shape[0]
+    assert 1 <= M <= MAX_ROWS, "gate_up_silu_rows is for at most 16 rows"
+    out = torch.empty(M, I, dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().ksa_gemm_rows_gate_up_silu(x2.data_ptr(), weight.data_ptr(), out.data_ptr(), M, I, K,
+                                                   x2.stride(0), weight.stride(0), I, _DT[x.dtype],
+                                                   _lib.stream_ptr(x.device))
+    _lib.check(rc, "ksa_gemm_rows_gate_up_silu")
+    return out.view(*x.shape[:-1], I)

@@ -141,10 +141,22 @@ class HipOps:
         self.silu_mul = elementwise.silu_mul
         self._decode = decode.ksa_decode
         self._linear_rows = gemm.linear_rows
+        self._gate_up_silu_rows = gemm.gate_up_silu_rows
         self._max_rows = gemm.MAX_ROWS
 
     def decode(self, q, kbuf, vbuf, start, end, scale):
         return self._decode(q, kbuf, vbuf, start, end, scale=scale)
+
+    def gate_up_act(self, x, weight):
+        """SiLU(x W_gate^T) * (x W_up^T) for the fused gate | up matrix: one kernel for the few rows of
+        a decode step, the library GEMM and the activation kernel otherwise."""
+        rows = x.numel() // x.shape[-1]
+        k = x.shape[-1]
+        if rows <= self._max_rows and k % 32 == 0 and rows * (k + 8) * 2 <= 160 * 1024:
+            return self._gate_up_silu_rows(x, weight)
+        if rows <= self._max_rows:
+            return self.silu_mul(self._linear_rows(x, weight, defer=True))
+        return self.silu_mul(F.linear(x, weight))
 
     def linear(self, x, weight, defer=False):
         """x W^T: the weight-streaming kernel for the few rows of a decode step, the library
@@ -284,8 +296,11 @@ class KsaQwen3ForCausalLM:
 
     def _mlp(self, lw, x, defer=False):
         """`defer`: the result only goes to `_add_norm` (see `HipOps.linear`)."""
-        gu = self.ops.linear(x, lw["gate_up_proj"], defer=defer)
-        return self.ops.linear(self.ops.silu_mul(gu), lw["down_proj"], defer=defer)
+        if hasattr(self.ops, "gate_up_act"):
+            act = self.ops.gate_up_act(x, lw["gate_up_proj"])
+        else:
+            act = self.ops.silu_mul(self.ops.linear(x, lw["gate_up_proj"], defer=defer))
+        return self.ops.linear(act, lw["down_proj"], defer=defer)
 
     def _logits(self, x_last, delta_last):
         _, h = self._add_norm(delta_last, x_last, self.w["norm"])
