@@ -202,6 +202,14 @@ int ksa_silu_mul(const void* gate, const void* up, void* out, long long rows, in
                  long long gate_row_stride, long long up_row_stride, long long out_row_stride,
                  int dtype, void* stream);
 
+/* out[r] = index of the largest value of row r (the lowest such index; a NaN counts as the largest
+ * value): the greedy token choice of a generation loop, torch.argmax(logits, dim=-1) of the
+ * generate() that drives the reference's model (the reference itself leaves it to transformers),
+ * in one small launch instead of the library's general reduction.  x [rows, N] of 16-bit values,
+ * row stride in elements (a multiple of 8), out [rows] int64. */
+int ksa_argmax_rows(const void* x, long long* out, int rows, int N, long long x_row_stride, int dtype,
+                    void* stream);
+
 /* ksa_silu_mul whose gate | up is still the K-split partial sums of the fused gate_up projection
  * (fp32 [ksplit][16][2 I], left by ksa_gemm_rows called with out == NULL): both halves are summed
  * in split order and rounded first, so the result is bit-identical to the two-kernel form.

@@ -39,6 +39,7 @@ _SIGNATURES = {
     "ksa_add_rmsnorm_partials": (_int, [_vp, _int] + [_vp] * 4 + [_int, _int] + [ctypes.c_longlong] * 3
                                  + [_int, ctypes.c_float, _vp]),
     "ksa_silu_mul": (_int, [_vp] * 3 + [ctypes.c_longlong, _int] + [ctypes.c_longlong] * 3 + [_int, _vp]),
+    "ksa_argmax_rows": (_int, [_vp, _vp, _int, _int, ctypes.c_longlong, _int, _vp]),
     "ksa_silu_mul_partials": (_int, [_vp, _int, _vp, _int, _int, ctypes.c_longlong, _int, _vp]),
     "ksa_gemm_rows_auto_splits": (_int, [_int, _int]),
     "ksa_gemm_rows_workspace_bytes": (ctypes.c_size_t, [_int, _int]),

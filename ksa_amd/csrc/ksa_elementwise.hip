@@ -211,6 +211,74 @@ __global__ __launch_bounds__(256) void ksa_silu_mul_kernel(const ActParams p) {
 
 bool al16(const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; }
 
+// ---- greedy token choice: index of the largest value of every row ----
+// One workgroup of 1024 threads per row; a thread scans every 1024th 16-byte item (several
+// requests in flight), then wave and workgroup reductions on (value, index) pairs.  Among equal
+// values the lowest index wins and a NaN counts as the largest value, as torch.argmax has it.
+struct ArgmaxParams {
+    const uint16_t* x;
+    long long* out;
+    int64_t xs;
+    int N;
+};
+
+__device__ __forceinline__ bool argmax_better(float a, int ia, float b, int ib) {
+    // (the library is built without NaN-honouring float compares: test the bits)
+    const bool na = (__builtin_bit_cast(uint32_t, a) & 0x7fffffffu) > 0x7f800000u;
+    const bool nb = (__builtin_bit_cast(uint32_t, b) & 0x7fffffffu) > 0x7f800000u;
+    if (na != nb) return na;
+    if (!na && a != b) return a > b;
+    return ia < ib;
+}
+
+template <typename T>
+__global__ __launch_bounds__(1024) void ksa_argmax_rows_kernel(const ArgmaxParams p) {
+    using C = KsaCvt<T>;
+    const uint16_t* row = p.x + (int64_t)blockIdx.x * p.xs;
+    float best = -INFINITY;
+    int bi = 0x7fffffff;
+    const int items = p.N / 8;
+    for (int j0 = threadIdx.x; j0 < items; j0 += 4 * 1024) {
+        u32x4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int j = j0 + 1024 * u;
+            v[u] = *reinterpret_cast<const u32x4*>(row + 8 * (j < items ? j : j0));
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int j = j0 + 1024 * u;
+            if (j < items) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float lo = C::up((uint16_t)(v[u][i] & 0xffffu)), hi = C::up((uint16_t)(v[u][i] >> 16));
+                    if (argmax_better(lo, 8 * j + 2 * i, best, bi)) best = lo, bi = 8 * j + 2 * i;
+                    if (argmax_better(hi, 8 * j + 2 * i + 1, best, bi)) best = hi, bi = 8 * j + 2 * i + 1;
+                }
+            }
+        }
+    }
+    for (int n = 8 * items + threadIdx.x; n < p.N; n += 1024) {  // a tail shorter than one item
+        const float v = C::up(row[n]);
+        if (argmax_better(v, n, best, bi)) best = v, bi = n;
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) {
+        const float ob = __shfl_xor(best, m);
+        const int oi = __shfl_xor(bi, m);
+        if (argmax_better(ob, oi, best, bi)) best = ob, bi = oi;
+    }
+    __shared__ float sv[16];
+    __shared__ int si[16];
+    if ((threadIdx.x & 63) == 0) sv[threadIdx.x >> 6] = best, si[threadIdx.x >> 6] = bi;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 16; ++w)
+            if (argmax_better(sv[w], si[w], best, bi)) best = sv[w], bi = si[w];
+        p.out[blockIdx.x] = bi;
+    }
+}
+
 }  // namespace
 
 extern "C" int ksa_add_rmsnorm(const void* x, const void* residual, const void* weight, void* out_norm,
@@ -300,5 +368,19 @@ extern "C" int ksa_silu_mul_partials(const float* partials, int ksplit, void* ou
     else
         hipLaunchKernelGGL((ksa_silu_mul_kernel<KsaF16, true>), dim3((unsigned)rows, yblocks), dim3(256), 0,
                            (hipStream_t)stream, p);
+    return ksa_check_launch();
+}
+
+extern "C" int ksa_argmax_rows(const void* x, long long* out, int rows, int N, long long x_row_stride,
+                               int dtype, void* stream) {
+    if (!x || !out) return KSA_ERR_NULL;
+    if (rows <= 0 || rows > 65535 || N <= 0) return KSA_ERR_INVALID;
+    if (dtype != KSA_DTYPE_BF16 && dtype != KSA_DTYPE_F16) return KSA_ERR_UNSUPPORTED;
+    if (!al16(x) || x_row_stride % 8) return KSA_ERR_ALIGN;
+    ArgmaxParams p{(const uint16_t*)x, out, x_row_stride, N};
+    if (dtype == KSA_DTYPE_BF16)
+        hipLaunchKernelGGL(ksa_argmax_rows_kernel<KsaBf16>, dim3(rows), dim3(1024), 0, (hipStream_t)stream, p);
+    else
+        hipLaunchKernelGGL(ksa_argmax_rows_kernel<KsaF16>, dim3(rows), dim3(1024), 0, (hipStream_t)stream, p);
     return ksa_check_launch();
 }

@@ -101,3 +101,16 @@ def silu_mul(gate, up: Optional[torch.Tensor] = None) -> torch.Tensor:
                                      u2.stride(0), out.stride(0), _DT[gate.dtype], _lib.stream_ptr(gate.device))
     _lib.check(rc, "ksa_silu_mul")
     return out.view(gate.shape)
+
+
+def argmax_rows(x: torch.Tensor) -> torch.Tensor:
+    """Index of the largest value along the last dimension (lowest index among equals), int64:
+    `torch.argmax(x, dim=-1)` for 16-bit logits in one small launch (`ksa_argmax_rows`)."""
+    assert x.is_cuda and x.dtype in _DT
+    x2 = _rows2d(x)
+    out = torch.empty(x2.shape[0], dtype=torch.long, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().ksa_argmax_rows(x2.data_ptr(), out.data_ptr(), x2.shape[0], x2.shape[1], x2.stride(0),
+                                        _DT[x.dtype], _lib.stream_ptr(x.device))
+    _lib.check(rc, "ksa_argmax_rows")
+    return out.view(x.shape[:-1])

@@ -142,10 +142,18 @@ class HipOps:
         self._decode = decode.ksa_decode
         self._linear_rows = gemm.linear_rows
         self._gate_up_silu_rows = gemm.gate_up_silu_rows
+        self._argmax_rows = elementwise.argmax_rows
         self._max_rows = gemm.MAX_ROWS
 
     def decode(self, q, kbuf, vbuf, start, end, scale):
         return self._decode(q, kbuf, vbuf, start, end, scale=scale)
+
+    def argmax(self, logits):
+        """Greedy token choice over the last dimension (lowest index among equal values)."""
+        if (logits.dtype in (torch.bfloat16, torch.float16) and logits.stride(-1) == 1 and logits.dim() == 2
+                and logits.stride(0) % 8 == 0 and logits.data_ptr() % 16 == 0):
+            return self._argmax_rows(logits)
+        return logits.argmax(-1)
 
     def gate_up_act(self, x, weight):
         """SiLU(x W_gate^T) * (x W_up^T) for the fused gate | up matrix: one kernel for the few rows of
@@ -403,7 +411,8 @@ class KsaQwen3ForCausalLM:
         per-step quantity (token ids, position, the cache row the new K/V go to, the attended row
         range) is read from device tensors of `st`, never baked into a launch."""
         cfg, ops = self.config, self.ops
-        cos, sin = self._rope_tables(st["pos"])
+        rope = st["rope_tab"].index_select(0, st["rope_rel"])   # [1, 2, D]: this step's cos and sin rows
+        cos, sin = rope[:, 0][None], rope[:, 1][None]
         x = self.w["embed_tokens"][st["tok"]]
         b = x.shape[0]
         delta = None
@@ -446,7 +455,6 @@ class KsaQwen3ForCausalLM:
         if st is None or st["batch"] != b or st["owner"] is not self:
             st = {"batch": b, "owner": self, "graph": None, "ptrs": None,
                   "tok": torch.zeros(b, 1, dtype=torch.long, device=self.device),
-                  "pos": torch.zeros(1, 1, dtype=torch.long, device=self.device),
                   # [kind: small / large window][destination row, range start, range end][sequence]
                   "cur": torch.zeros(2, 3, b, dtype=torch.int32, device=self.device)}
             cache._ksa_graph_state = st
@@ -466,11 +474,39 @@ class KsaQwen3ForCausalLM:
                 a, e = cache.attention_range(li)
                 vals[kind] = [rows[kind], a, e]
                 rows[kind] = None
-        # a fresh pageable host tensor: the runtime stages it before the call returns, so the host
-        # may run ahead of the GPU without overwriting values of a step still in flight
-        st["cur"].copy_(torch.tensor(vals, dtype=torch.int32).view(2, 3, 1))
+        # The values travel through a ring of pinned host slots: a copy from pageable memory would
+        # hold the host until the GPU has reached it, i.e. until the previous step has ended, and
+        # the GPU would then idle while the host prepares the next replay.  A slot is written again
+        # only after the copy that read it has run (its event), so the host may be up to a ring's
+        # length of steps ahead of the GPU.
+        if "ring" not in st:
+            st["ring"] = torch.empty(16, 2, 3, b, dtype=torch.int32, pin_memory=True)
+            st["ring_events"] = [None] * 16
+            st["ring_next"] = 0
+        slot = st["ring_next"]
+        st["ring_next"] = (slot + 1) % 16
+        if st["ring_events"][slot] is not None:
+            st["ring_events"][slot].synchronize()
+        st["ring"][slot].copy_(torch.tensor(vals, dtype=torch.int32).view(2, 3, 1))
+        st["cur"].copy_(st["ring"][slot], non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record(torch.cuda.current_stream(self.device))
+        st["ring_events"][slot] = ev
         st["tok"].copy_(token_ids.to(self.device))
-        st["pos"].fill_(p)
+        # rotary rows of a window of positions, made with the prefill's own tensor ops (so a step's
+        # cos / sin are the values `_rope_tables` gives) and refilled in place when p leaves it; the
+        # recorded step only picks a row
+        if st.get("rope_p0") is None or not (st["rope_p0"] <= p < st["rope_p0"] + st["rope_tab"].shape[0]):
+            n = 1024
+            c, s_ = self._rope_tables(torch.arange(p, p + n, device=self.device)[None])
+            tab = torch.stack((c[0], s_[0]), dim=1)
+            if "rope_tab" in st:
+                st["rope_tab"].copy_(tab)
+            else:
+                st["rope_tab"] = tab.contiguous()
+                st["rope_rel"] = torch.zeros(1, dtype=torch.long, device=self.device)
+            st["rope_p0"] = p
+        st["rope_rel"].fill_(p - st["rope_p0"])
         ptrs = tuple((t.data_ptr(), tuple(t.shape), t.stride()) for t in cache.key_cache + cache.value_cache)
         if st["graph"] is None or st["ptrs"] != ptrs:
             side = torch.cuda.Stream(device=self.device)
@@ -505,7 +541,8 @@ class KsaQwen3ForCausalLM:
         for t in range(max_new_tokens):
             if return_logits:
                 steps.append(logits[:, 0].float())
-            nxt = logits[:, 0].argmax(-1, keepdim=True)
+            last = logits[:, 0]
+            nxt = (self.ops.argmax(last) if hasattr(self.ops, "argmax") else last.argmax(-1))[:, None]
             out.append(nxt)
             if t + 1 < max_new_tokens:
                 feed = nxt if forced is None else forced[:, t:t + 1].to(self.device)

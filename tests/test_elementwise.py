@@ -100,3 +100,33 @@ def test_gpu_silu_mul(dtype, rows, I):
     gug = gu.cuda()
     got = silu_mul(gug[:, :I], gug[:, I:])
     _ulp_check(got, exp, 5e-3)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,N", [(8, 151936), (1, 8), (3, 1000), (5, 8192 + 3), (16, 5)])
+def test_gpu_argmax_rows(dtype, rows, N):
+    """The greedy token choice against torch.argmax on the CPU (first index among equal values:
+    16-bit logits tie often), with the row maximum planted at both ends, inside a tail that is
+    shorter than one 16-byte item, and doubled."""
+    from ksa_amd.elementwise import argmax_rows
+    g = torch.Generator().manual_seed(rows * 1000 + N)
+    Np = (N + 7) // 8 * 8
+    x = torch.randn(rows, Np, generator=g).to(dtype)[:, :N]   # rows start 16-byte aligned
+    x[0, N - 1] = 30.0
+    if rows > 1:
+        x[1, 0] = 30.0
+    if rows > 2:
+        x[2, N // 2] = 30.0
+        x[2, N - 1] = 30.0                                    # the first of two equal maxima wins
+    def dev(t):  # same padded row stride on the GPU (a plain .cuda() would pack the rows)
+        buf = torch.zeros(rows, Np, dtype=dtype, device="cuda")
+        buf[:, :N] = t
+        return buf[:, :N]
+
+    got = argmax_rows(dev(x)).cpu()
+    want = x.float().argmax(-1)
+    assert got.dtype == torch.long and torch.equal(got, want), (got, want)
+    if rows > 3 and N > 20:
+        x[3, 17] = float("nan")                               # a NaN counts as the largest value
+        assert int(argmax_rows(dev(x))[3]) == 17 == int(x.float().argmax(-1)[3])
