@@ -246,6 +246,34 @@ int ksa_gemm_rows_gate_up_silu(const void* x, const void* w, void* out, int M, i
                                long long x_row_stride, long long w_row_stride, long long out_row_stride,
                                int dtype, void* stream);
 
+/* The MLP of a decoder layer for at most 16 rows as one launch that holds the workgroups of both
+ * products; those of the down projection request their weights and then wait for the tiles of the
+ * activation they need, which the gate | up workgroups count off in device memory (Qwen3MLP.forward,
+ * HF:507-514):
+ *   a = SiLU(x W_gate^T) * (x W_up^T)                        (like ksa_gemm_rows_gate_up_silu)
+ *   down_partials[c] = a[:, 512 c : 512 c + 512] W_down[:, same]^T   for c < ksa_mlp_rows_down_splits(H, I)
+ *   = ceil(I / 512),
+ * i.e. the down projection as K-split partial sums [splits][16][H] fp32 for a consumer that adds
+ * them (ksa_add_rmsnorm_partials).  Takes the place of ksa_gemm_rows_gate_up_silu + ksa_gemm_rows:
+ * the weights of the down projection move while the activation is still being made, and no launch
+ * ramp lies between the two products.
+ *   x [M, H]; w_gate_up [2 I, H]; w_down [H, I]; H a multiple of 128 with M (H + 8) 2 bytes within
+ *   160 KiB of LDS, I a multiple of 32 up to 30720; row strides in elements, multiples of 8.
+ *   workspace: ksa_mlp_rows_workspace_bytes(H, I) bytes, 16-byte aligned, ZEROED ONCE by the caller
+ *   before its first use and then left alone (its counting words go up from launch to launch);
+ *   it belongs to one device and one pair (H, I), and launches that share it must not overlap.
+ *   Every wait inside the kernel is bounded: a workgroup that does not see its tiles arrive within
+ *   about a second gives up, the output of that launch is unusable and the 8-byte word at
+ *   ksa_mlp_rows_status_offset() of the workspace reads 1 - the caller then zeroes the workspace
+ *   again.  KSA_ERR_UNSUPPORTED for sizes outside the above: use
+ *   the two separate calls. */
+int ksa_mlp_rows_down_splits(int H, int I);
+size_t ksa_mlp_rows_workspace_bytes(int H, int I);
+size_t ksa_mlp_rows_status_offset(void);
+int ksa_mlp_rows(const void* x, const void* w_gate_up, const void* w_down, float* down_partials, int M, int H,
+                 int I, long long x_row_stride, long long w_gate_up_row_stride, long long w_down_row_stride,
+                 int dtype, void* workspace, size_t workspace_bytes, void* stream);
+
 /* Host-side diagnostic: number of key columns in [a, b) visible to query row q under the
  * closed-form rule the kernels use (no GPU involved). */
 long long ksa_debug_count_visible(long long q, long long a, long long b, int C, int S, int W,

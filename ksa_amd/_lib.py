@@ -45,6 +45,10 @@ _SIGNATURES = {
     "ksa_gemm_rows_workspace_bytes": (ctypes.c_size_t, [_int, _int]),
     "ksa_gemm_rows": (_int, [_vp] * 3 + [_int] * 3 + [ctypes.c_longlong] * 3 + [_int, _int, _vp, ctypes.c_size_t, _vp]),
     "ksa_gemm_rows_gate_up_silu": (_int, [_vp] * 3 + [_int] * 3 + [ctypes.c_longlong] * 3 + [_int, _vp]),
+    "ksa_mlp_rows_down_splits": (_int, [_int, _int]),
+    "ksa_mlp_rows_workspace_bytes": (ctypes.c_size_t, [_int, _int]),
+    "ksa_mlp_rows_status_offset": (ctypes.c_size_t, []),
+    "ksa_mlp_rows": (_int, [_vp] * 4 + [_int] * 3 + [ctypes.c_longlong] * 3 + [_int, _vp, ctypes.c_size_t, _vp]),
     "ksa_debug_count_visible": (ctypes.c_longlong, [ctypes.c_longlong] * 3 + [_int] * 7),
 }
 

@@ -10,7 +10,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libksa_hip.so")
 SOURCES = ["ksa_api.hip", "ksa_index.hip", "ksa_prefill.hip", "ksa_decode.hip", "ksa_cache.hip",
-           "ksa_pre.hip", "ksa_elementwise.hip", "ksa_gemm_rows.hip"]
+           "ksa_pre.hip", "ksa_elementwise.hip", "ksa_gemm_rows.hip", "ksa_mlp_rows.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

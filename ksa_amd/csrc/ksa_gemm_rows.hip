@@ -13,10 +13,9 @@
 
 #include "ksa_api_internal.h"
 #include "ksa_cvt.h"
+#include "ksa_rows_mfma.h"
 
 namespace {
-
-typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 struct GemmParams {
     const uint16_t* x;   // [M, K], row stride xs
@@ -26,25 +25,6 @@ struct GemmParams {
     int64_t xs, ws, os;
     int M, N, K, ksplit;
 };
-
-template <typename T>
-__device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c);
-template <>
-__device__ __forceinline__ f32x4 mfma16<KsaBf16>(u32x4 a, u32x4 b, f32x4 c) {
-    typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
-                                                   0, 0, 0);
-}
-template <>
-__device__ __forceinline__ f32x4 mfma16<KsaF16>(u32x4 a, u32x4 b, f32x4 c) {
-    typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c,
-                                                  0, 0, 0);
-}
-
-constexpr int kChunkSteps = 16;                 // K steps (of 32) per staged chunk of x
-constexpr int kChunkK = 32 * kChunkSteps;       // 512 elements of K
-constexpr int kRowB = (kChunkK + 8) * 2;        // padded LDS row of x in bytes (conflict-free b128 reads)
 
 // grid: (tiles of 64 output columns, K splits); block: 4 waves, each 16 columns over the whole K
 // slice.  Per chunk of 512 K elements a wave first requests its 16 weight fragments (16 x 16

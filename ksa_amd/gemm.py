@@ -79,3 +79,51 @@ def gate_up_silu_rows(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
                                                    _lib.stream_ptr(x.device))
     _lib.check(rc, "ksa_gemm_rows_gate_up_silu")
     return out.view(*x.shape[:-1], I)
+
+
+class MlpRowsWorkspace:
+    """Barrier words and the activation buffer of `mlp_rows` for one (device, hidden size, MLP size):
+    zeroed once, then shared by every layer's call on that stream (the calls run one after the other)."""
+
+    def __init__(self, H: int, I: int, device):
+        L = _lib.lib()
+        self.H, self.I = H, I
+        self.buf = torch.zeros(L.ksa_mlp_rows_workspace_bytes(H, I), dtype=torch.uint8, device=device)
+        self._status = self.buf[L.ksa_mlp_rows_status_offset():][:8].view(torch.int64)
+
+    def failed(self) -> bool:
+        """True if a launch gave up waiting at a grid barrier (synchronises; the workspace is zeroed
+        again so that it can be used further)."""
+        bad = bool(self._status.item() != 0)
+        if bad:
+            self.buf.zero_()
+        return bad
+
+
+def mlp_rows_supported(M: int, H: int, I: int) -> bool:
+    return (1 <= M <= MAX_ROWS and H % 128 == 0 and I % 32 == 0 and I <= 30720
+            and M * (H + 8) * 2 <= 160 * 1024)
+
+
+def mlp_rows(x: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor, ws: MlpRowsWorkspace) -> SplitKPartials:
+    """One launch for `down(SiLU(gate(x)) * up(x))` at a decode step (`ksa_mlp_rows`;
+    modeling_qwen3sa.py:507-514).  The result comes as `SplitKPartials` for the next residual add + norm."""
+    H = x.shape[-1]
+    I = w_gate_up.shape[0] // 2
+    dt = x.dtype
+    assert x.is_cuda and dt in _DT
+    assert w_gate_up.shape == (2 * I, H) and w_down.shape == (H, I) and w_gate_up.dtype == dt and w_down.dtype == dt
+    assert w_gate_up.stride(1) == 1 and w_down.stride(1) == 1 and ws.H == H and ws.I == I
+    x2 = x.reshape(-1, H)
+    if x2.stride(1) != 1:
+        x2 = x2.contiguous()
+    M = x2.shape[0]
+    L = _lib.lib()
+    with torch.cuda.device(x2.device):
+        ks = L.ksa_mlp_rows_down_splits(H, I)
+        part = torch.empty(ks * 16 * H, dtype=torch.float32, device=x2.device)
+        rc = L.ksa_mlp_rows(x2.data_ptr(), w_gate_up.data_ptr(), w_down.data_ptr(), part.data_ptr(), M, H, I,
+                            x2.stride(0), w_gate_up.stride(0), w_down.stride(0), _DT[dt], ws.buf.data_ptr(),
+                            ws.buf.numel(), _lib.stream_ptr(x2.device))
+    _lib.check(rc, "ksa_mlp_rows")
+    return SplitKPartials(part.view(torch.uint8), ks, M, x.shape, dt)

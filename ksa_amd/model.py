@@ -144,6 +144,8 @@ class HipOps:
         self._gate_up_silu_rows = gemm.gate_up_silu_rows
         self._argmax_rows = elementwise.argmax_rows
         self._max_rows = gemm.MAX_ROWS
+        self._gemm = gemm
+        self._mlp_ws = {}   # (device, H, I) -> MlpRowsWorkspace, see `mlp_rows`
 
     def decode(self, q, kbuf, vbuf, start, end, scale):
         return self._decode(q, kbuf, vbuf, start, end, scale=scale)
@@ -154,6 +156,27 @@ class HipOps:
                 and logits.stride(0) % 8 == 0 and logits.data_ptr() % 16 == 0):
             return self._argmax_rows(logits)
         return logits.argmax(-1)
+
+    def prepare_mlp_rows(self, H, I, device):
+        """Makes the workspace of `mlp_rows` for this MLP shape ahead of time (it has to exist, zeroed,
+        before a step that uses it is recorded into a graph)."""
+        key = (str(device), H, I)
+        if key not in self._mlp_ws:
+            self._mlp_ws[key] = self._gemm.MlpRowsWorkspace(H, I, device)
+        return self._mlp_ws[key]
+
+    def mlp_rows(self, x, w_gate_up, w_down):
+        """down(SiLU(gate(x)) * up(x)) for the few rows of a decode step in one launch, as the K-split
+        partial sums of the down projection; None when the shape is outside what that kernel takes."""
+        rows = x.numel() // x.shape[-1]
+        H, I = x.shape[-1], w_down.shape[1]
+        if not self._gemm.mlp_rows_supported(rows, H, I):
+            return None
+        return self._gemm.mlp_rows(x, w_gate_up, w_down, self.prepare_mlp_rows(H, I, x.device))
+
+    def mlp_rows_failed(self):
+        """True if a `mlp_rows` launch gave up waiting (synchronises); see `MlpRowsWorkspace.failed`."""
+        return any(ws.failed() for ws in self._mlp_ws.values())
 
     def gate_up_act(self, x, weight):
         """SiLU(x W_gate^T) * (x W_up^T) for the fused gate | up matrix: one kernel for the few rows of
@@ -254,6 +277,8 @@ class KsaQwen3ForCausalLM:
         self.dtype, self.device = emb.dtype, emb.device
         self.inv_freq_dev = self.inv_freq.to(self.device)
         self.lm_head = emb[: config.vocab_size] if config.tie_word_embeddings else weights["lm_head"]
+        if hasattr(self.ops, "prepare_mlp_rows") and self.device.type == "cuda":
+            self.ops.prepare_mlp_rows(config.hidden_size, config.intermediate_size, self.device)
 
     # ---- pieces ----------------------------------------------------------------------
     def _add_norm(self, delta, x, w):
@@ -304,6 +329,10 @@ class KsaQwen3ForCausalLM:
 
     def _mlp(self, lw, x, defer=False):
         """`defer`: the result only goes to `_add_norm` (see `HipOps.linear`)."""
+        if defer and hasattr(self.ops, "mlp_rows"):
+            out = self.ops.mlp_rows(x, lw["gate_up_proj"], lw["down_proj"])
+            if out is not None:
+                return out
         if hasattr(self.ops, "gate_up_act"):
             act = self.ops.gate_up_act(x, lw["gate_up_proj"])
         else:
@@ -548,4 +577,7 @@ class KsaQwen3ForCausalLM:
                 feed = nxt if forced is None else forced[:, t:t + 1].to(self.device)
                 logits = self.decode_step_graph(feed, cache) if use_graph else self.decode_step(feed, cache)
         ids = torch.cat([input_ids.to(self.device)] + out, dim=1)
+        if hasattr(self.ops, "mlp_rows_failed") and self.ops.mlp_rows_failed():
+            raise RuntimeError("ksa_mlp_rows: a workgroup gave up waiting for the activation tiles of its chunk; "
+                               "the tokens of this call are not valid")
         return (ids, torch.stack(steps, dim=1)) if return_logits else ids

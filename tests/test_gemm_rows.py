@@ -122,3 +122,44 @@ def test_gpu_gate_up_silu_one_launch(dtype, M, I, K):
     assert (a != b).float().mean() <= 0.02
     two = silu_mul(linear_rows(x.cuda(), w.cuda()))
     assert (two[0].float().cpu() != a).float().mean() <= 0.02
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,H,I", [(8, 2560, 9728), (1, 2560, 9728), (16, 1024, 768), (3, 256, 256), (5, 4096, 512),
+                                   (8, 768, 2304)])
+def test_gpu_mlp_rows_one_launch(dtype, M, H, I):
+    """The MLP of a layer in one launch of resident workgroups (gate | up + SiLU -> grid barrier ->
+    down) against the two separate launches it stands for: the down projection, added up from its
+    partial sums, equal to the separate path's to within the few 16-bit units that a different
+    split of K allows, and close to the fp64 product of the 16-bit activation the separate path
+    makes (the activation itself is computed in the same order in both).  Run three times on one
+    workspace (the barrier words count on), the last time after another shape has used a workspace
+    of its own."""
+    from ksa_amd import silu_mul
+    from ksa_amd.gemm import MlpRowsWorkspace, gate_up_silu_rows, linear_rows, mlp_rows
+    g = torch.Generator().manual_seed(M * 7 + H + I)
+    dev = torch.device("cuda")
+    h = torch.randn(1, M, H, generator=g).to(dtype).to(dev)
+    w_gu = (torch.randn(2 * I, H, generator=g) * 0.04).to(dtype).to(dev)
+    w_dn = (torch.randn(H, I, generator=g) * 0.03).to(dtype).to(dev)
+    act = gate_up_silu_rows(h, w_gu) if M * (H + 8) * 2 <= 160 * 1024 else silu_mul(linear_rows(h, w_gu))
+    d_ref = linear_rows(act, w_dn)
+    want = (act[0].double() @ w_dn.double().T)
+    ws = MlpRowsWorkspace(H, I, dev)
+    for rep in range(3):
+        if rep == 2:
+            ws_other = MlpRowsWorkspace(256, 512, dev)
+            mlp_rows(torch.ones(1, 2, 256, dtype=dtype, device=dev), torch.ones(1024, 256, dtype=dtype, device=dev),
+                     torch.ones(256, 512, dtype=dtype, device=dev), ws_other)
+            assert not ws_other.failed()
+        d_part = mlp_rows(h, w_gu, w_dn, ws)
+        torch.cuda.synchronize()
+        assert not ws.failed(), "a workgroup gave up at the grid barrier"
+        parts = d_part.workspace.view(torch.float32).view(d_part.ksplit, 16, H)[:, :M]
+        d_new = parts.sum(0).to(dtype)
+        err = (parts.double().sum(0) - want).abs().max().item()
+        assert err <= 2e-3 * want.abs().max().item() + 1e-4, err
+        ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
+        diff = (d_new.float() - d_ref[0].float()).abs()
+        assert (diff <= 2 * ulp * d_ref[0].float().abs() + 4 * ulp * want.abs().max().item() * 2.0 ** -6).all(), diff.max()
