@@ -67,13 +67,13 @@ __device__ __forceinline__ unsigned long long add_agent(unsigned long long* p, u
 }
 // 16 bytes written by another workgroup of this launch: a load that is not served from this XCD's
 // L2 (the cache-control bit the compiler sets for agent-scope atomic loads; those stop at 8 bytes).
-// Assembly, so the compiler does not know of the request: ld_agent_wait() before the value is used.
-__device__ __forceinline__ u32x4 ld_agent_x4(const void* p) {
+// Assembly with the wait inside the statement: the compiler does not know that the value of a bare
+// asm load is still on its way and may copy the register before it has arrived.
+__device__ __forceinline__ u32x4 ld_agent_x4_wait(const void* p) {
     u32x4 v;
-    asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v) : "v"(p) : "memory");
+    asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
     return v;
 }
-__device__ __forceinline__ void ld_agent_wait() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 template <typename T>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(6, 6))) void ksa_mlp_rows_kernel(const MlpParams p) {
@@ -200,9 +200,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
         const int per_row = nst * 4;  // 16-byte items
         for (int e = tid; e < p.M * per_row; e += (int)blockDim.x) {  // (M = 8: one item per thread)
             const int m = e / per_row, j = e - m * per_row;
-            const u32x4 v = ld_agent_x4(reinterpret_cast<const u32x4*>(p.act + (int64_t)m * (p.I / 4) + s0c * 8) + j);
-            ld_agent_wait();
-            *reinterpret_cast<u32x4*>(lds + m * kRowB + 16 * j) = v;
+            *reinterpret_cast<u32x4*>(lds + m * kRowB + 16 * j) =
+                ld_agent_x4_wait(reinterpret_cast<const u32x4*>(p.act + (int64_t)m * (p.I / 4) + s0c * 8) + j);
         }
         __syncthreads();
         if (live) {
