@@ -258,7 +258,7 @@ int ksa_gemm_rows_gate_up_silu(const void* x, const void* w, void* out, int M, i
  * the weights of the down projection move while the activation is still being made, and no launch
  * ramp lies between the two products.
  *   x [M, H]; w_gate_up [2 I, H]; w_down [H, I]; H a multiple of 128 with M (H + 8) 2 bytes within
- *   160 KiB of LDS, I a multiple of 32 up to 30720; row strides in elements, multiples of 8.
+ *   160 KiB of LDS, I a multiple of 32 up to 26624; row strides in elements, multiples of 8.
  *   workspace: ksa_mlp_rows_workspace_bytes(H, I) bytes, 16-byte aligned, ZEROED ONCE by the caller
  *   before its first use and then left alone (its counting words go up from launch to launch);
  *   it belongs to one device and one pair (H, I), and launches that share it must not overlap.
@@ -273,6 +273,19 @@ size_t ksa_mlp_rows_status_offset(void);
 int ksa_mlp_rows(const void* x, const void* w_gate_up, const void* w_down, float* down_partials, int M, int H,
                  int I, long long x_row_stride, long long w_gate_up_row_stride, long long w_down_row_stride,
                  int dtype, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ksa_mlp_rows with the residual add + RMSNorm in front of the MLP in the same launch (HF:944-947):
+ *   out_sum = residual + round(sum of the o_proj partial sums),  x = RMSNorm(out_sum) * norm_weight
+ * by one workgroup per row at the head of the grid (arithmetic and summation order of
+ * ksa_add_rmsnorm_partials; out_sum bit-identical, x to one unit in the last place), for whose rows
+ * the gate | up workgroups wait with their first weights already requested.  Takes the place of
+ * ksa_add_rmsnorm_partials + ksa_mlp_rows.  o_partials [o_ksplit][16][H] fp32 (ksa_gemm_rows with a
+ * null output); residual, out_sum [M, H]; H up to 4096; the rest as ksa_mlp_rows, same workspace. */
+int ksa_add_rmsnorm_mlp_rows(const float* o_partials, int o_ksplit, const void* residual, const void* norm_weight,
+                             void* out_sum, const void* w_gate_up, const void* w_down, float* down_partials, int M,
+                             int H, int I, long long residual_row_stride, long long sum_row_stride,
+                             long long w_gate_up_row_stride, long long w_down_row_stride, int dtype, float eps,
+                             void* workspace, size_t workspace_bytes, void* stream);
 
 /* Host-side diagnostic: number of key columns in [a, b) visible to query row q under the
  * closed-form rule the kernels use (no GPU involved). */

@@ -49,6 +49,8 @@ _SIGNATURES = {
     "ksa_mlp_rows_workspace_bytes": (ctypes.c_size_t, [_int, _int]),
     "ksa_mlp_rows_status_offset": (ctypes.c_size_t, []),
     "ksa_mlp_rows": (_int, [_vp] * 4 + [_int] * 3 + [ctypes.c_longlong] * 3 + [_int, _vp, ctypes.c_size_t, _vp]),
+    "ksa_add_rmsnorm_mlp_rows": (_int, [_vp, _int] + [_vp] * 6 + [_int] * 3 + [ctypes.c_longlong] * 4
+                                 + [_int, ctypes.c_float, _vp, ctypes.c_size_t, _vp]),
     "ksa_debug_count_visible": (ctypes.c_longlong, [ctypes.c_longlong] * 3 + [_int] * 7),
 }
 

@@ -20,6 +20,12 @@
 // follow as places become free.  No grid-wide barrier, no need for the grid to be resident as a
 // whole, and the workgroups stay short-lived (which streams faster here than workgroups that loop).
 //
+// Optionally the launch begins with the residual add + RMSNorm in front of the MLP (one workgroup per
+// row, on the K-split partial sums of the o projection: modeling_qwen3sa.py:944-947), and the
+// gate | up workgroups, their first weights requested, wait for its rows the same way - the norm's
+// chain of dependent memory trips then runs next to the first weight requests instead of in a
+// launch of its own.
+//
 // The activation, which one workgroup writes and another reads inside the launch, goes through
 // agent-scope atomic stores and cache-bypassing loads (the L2 caches of the eight XCDs are not
 // coherent with each other for plain accesses); weights, input and output use plain accesses.
@@ -38,13 +44,24 @@ namespace {
 
 constexpr int kSlices = 4;        // K slices of the hidden size = waves per gate / up half
 constexpr int kWordStride = 64;   // 64-bit words are 512 bytes apart
-// words: [0] launches so far, [1] down workgroups done, [2] status, [4 + c] tiles of chunk c stored
-constexpr int kWordLaunches = 0, kWordDone = 1, kWordStatus = 2, kWordChunk0 = 4;
-constexpr int kMaxChunks = 60;    // K of the down projection up to 30720
+// words: [0] launches so far, [1] down workgroups done, [2] status, [4 .. 11] rows of the norm stage done
+// (eight copies, a gate | up workgroup watches copy number % 8: hundreds of workgroups polling one
+// word would queue at it), [12 + c] tiles of chunk c stored
+constexpr int kWordLaunches = 0, kWordDone = 1, kWordStatus = 2, kWordHeadLaunches = 3, kWordHead0 = 4, kHeadCopies = 8,
+              kWordChunk0 = 12;  // ([3] launches with a norm stage: those without one do not move the words [4 .. 11])
+constexpr int kMaxChunks = 52;    // K of the down projection up to 26624
 constexpr int kSyncWords = kWordStride * (kWordChunk0 + kMaxChunks);
 
 struct MlpParams {
-    const uint16_t* x;        // h rows [M][H]
+    const uint16_t* x;        // h rows [M][H]; null: they come from the norm stage of this launch
+    const float* o_part;      // norm stage: [o_ksplit][16][H] partial sums of the o projection
+    const uint16_t* res;      // norm stage: residual rows [M][H]
+    const uint16_t* norm_w;   // norm stage: weight [H]
+    uint16_t* out_sum;        // norm stage: residual + o projection [M][H]
+    unsigned long long* hbuf; // norm stage: its rows for the gate | up workgroups, [M][H / 4]
+    int64_t res_rs, sum_rs;
+    int o_ksplit, head;       // head: workgroups of the norm stage (M, or 0)
+    float eps;
     const uint16_t* w_gu;     // [2 I][H]
     const uint16_t* w_dn;     // [H][I]
     float* dn_part;           // [KC][16][H]
@@ -82,7 +99,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
     __shared__ int s_fail;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: what depends on it stays in scalar registers
     const int r = lane & 15;
     const int kq = lane >> 4;
     const int xrow = min(r, p.M - 1);
@@ -90,9 +107,74 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
     u32x4 a[kB];
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 
-    if ((int)blockIdx.x < p.UB) {
+    if ((int)blockIdx.x < p.head) {
+        // ---- norm stage, one workgroup per row: x' = residual + sum of the o_proj partial sums (plain
+        // store, for later launches), h = norm(x') w (for the gate | up workgroups of this launch).
+        // Arithmetic and summation order of ksa_add_rmsnorm_partials. ----
+        const int row = blockIdx.x;
+        const int items = p.H / 8;  // at most 512: one per thread
+        float* s_ss = reinterpret_cast<float*>(lds);
+        float ss = 0.f;
+        u32x4 rsum = {0u, 0u, 0u, 0u}, wv = {0u, 0u, 0u, 0u};
+        if (tid < items) {
+            wv = *reinterpret_cast<const u32x4*>(p.norm_w + 8 * tid);
+            const u32x4 q = *reinterpret_cast<const u32x4*>(p.res + (int64_t)row * p.res_rs + 8 * tid);
+            float ac[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            for (int sp0 = 0; sp0 < p.o_ksplit; sp0 += 4) {  // (four slices requested at a time: registers)
+                f32x4 lo[4], hi[4];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const float* src = p.o_part + ((int64_t)min(sp0 + k, p.o_ksplit - 1) * 16 + row) * p.H + 8 * tid;
+                    lo[k] = *reinterpret_cast<const f32x4*>(src);
+                    hi[k] = *reinterpret_cast<const f32x4*>(src + 4);
+                }
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    if (sp0 + k < p.o_ksplit) {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) ac[i] += lo[k][i], ac[4 + i] += hi[k][i];
+                    }
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t x = C::down2(ac[2 * i], ac[2 * i + 1]);
+                rsum[i] = C::down2(C::lo(x) + C::lo(q[i]), C::hi(x) + C::hi(q[i]));
+                const float a_ = C::lo(rsum[i]), b_ = C::hi(rsum[i]);
+                ss = fmaf(a_, a_, ss);
+                ss = fmaf(b_, b_, ss);
+            }
+            *reinterpret_cast<u32x4*>(p.out_sum + (int64_t)row * p.sum_rs + 8 * tid) = rsum;
+        }
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1) ss += __shfl_xor(ss, m);
+        if (lane == 0) s_ss[wave] = ss;
+        __syncthreads();
+        ss = 0.f;
+        for (int w = 0; w < (items + 63) / 64; ++w) ss += s_ss[w];
+        const float inv = rsqrtf(ss / (float)p.H + p.eps);
+        if (tid < items) {
+            uint32_t o[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t y = C::down2(C::lo(rsum[i]) * inv, C::hi(rsum[i]) * inv);
+                o[i] = C::down2(C::lo(wv[i]) * C::lo(y), C::hi(wv[i]) * C::hi(y));
+            }
+            unsigned long long* hp = p.hbuf + (int64_t)row * (p.H / 4) + 2 * tid;
+            st_agent(hp, (unsigned long long)o[0] | ((unsigned long long)o[1] << 32));
+            st_agent(hp + 1, (unsigned long long)o[2] | ((unsigned long long)o[3] << 32));
+        }
+        __syncthreads();  // every store of the workgroup is issued and counted off (s_waitcnt before the barrier)
+        if (tid < kHeadCopies) {
+            __builtin_amdgcn_s_waitcnt(0);
+            add_agent(p.sync + kWordStride * (kWordHead0 + tid), 1ull);
+        }
+        return;
+    }
+    const int bid = blockIdx.x - p.head;  // number among the workgroups of the two products
+    if (bid < p.UB) {
         // ---- 16 columns of the activation (ksa_gemm_gate_up_silu_kernel's scheme) ----
-        const int u = blockIdx.x;
+        const int u = bid;
         const int half = wave / kSlices;  // 0: gate rows of w, 1: up rows
         const int slice = wave - half * kSlices;
         const int sl_steps = p.H / 32 / kSlices;  // K steps of a slice (H is a multiple of 128)
@@ -103,12 +185,44 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
 #pragma unroll
             for (int k = 0; k < kB; ++k) a[k] = *reinterpret_cast<const u32x4*>(wp + 32 * min(s0 + k, sl_steps - 1));
         };
-        load_steps(0);  // in flight while x is staged
-        const int per_row = p.H / 8;
-        for (int e = tid; e < p.M * per_row; e += blockDim.x) {
-            const int m = e / per_row, j = e - m * per_row;
-            *reinterpret_cast<u32x4*>(lds + m * rowb + 16 * j) =
-                *reinterpret_cast<const u32x4*>(p.x + (int64_t)m * p.x_rs + 8 * j);
+        load_steps(0);  // in flight while x is waited for and staged
+        if (p.head > 0) {
+            // the rows of the norm stage: wait for its count, then fetch them past this XCD's L2
+            if (tid == 0) {
+                const unsigned long long launch = ld_agent(p.sync + kWordStride * kWordHeadLaunches);
+                unsigned long long* word = p.sync + kWordStride * (kWordHead0 + (bid % kHeadCopies));
+                unsigned long long* status = p.sync + kWordStride * kWordStatus;
+                const unsigned long long want = (launch + 1) * (unsigned long long)p.head;
+                unsigned spins = 0;
+                int fail = 0;
+                while (ld_agent(word) < want) {
+                    __builtin_amdgcn_s_sleep(4);
+                    if (++spins > p.spin_limit) {
+                        st_agent(status, 1ull);
+                        fail = 1;
+                        break;
+                    }
+                    if ((spins & 63) == 0 && ld_agent(status) != 0) {
+                        fail = 1;
+                        break;
+                    }
+                }
+                s_fail = fail;
+            }
+            __syncthreads();
+            if (s_fail) return;
+            const int per_row = p.H / 4;  // 8-byte words (agent-scope loads the compiler tracks: several in flight)
+            for (int e = tid; e < p.M * per_row; e += blockDim.x) {
+                const int m = e / per_row, j = e - m * per_row;
+                *reinterpret_cast<unsigned long long*>(lds + m * rowb + 8 * j) = ld_agent(p.hbuf + (int64_t)m * per_row + j);
+            }
+        } else {
+            const int per_row = p.H / 8;
+            for (int e = tid; e < p.M * per_row; e += blockDim.x) {
+                const int m = e / per_row, j = e - m * per_row;
+                *reinterpret_cast<u32x4*>(lds + m * rowb + 16 * j) =
+                    *reinterpret_cast<const u32x4*>(p.x + (int64_t)m * p.x_rs + 8 * j);
+            }
         }
         __syncthreads();
         for (int s0 = 0; s0 < sl_steps; s0 += kB) {
@@ -152,7 +266,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
     }
 
     // ---- one 512-element chunk kc of the down projection's K for the column tiles of group grp ----
-    const int d = blockIdx.x - p.UB;
+    const int d = bid - p.UB;
     const int kc = d / p.GR, grp = d - kc * p.GR;
     constexpr int W = 2 * kSlices;
     const int CT = p.H / 16;
@@ -198,7 +312,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
     if (s_fail == 0) {
         // the chunk of the activation: [M][512] through cache-bypassing loads into LDS
         const int per_row = nst * 4;  // 16-byte items
-        for (int e = tid; e < p.M * per_row; e += (int)blockDim.x) {  // (M = 8: one item per thread)
+        int t1 = tid;  // (an opaque copy: what is derived from it does not live across the wait above)
+        asm volatile("" : "+v"(t1));
+        for (int e = t1; e < p.M * per_row; e += (int)blockDim.x) {  // (M = 8: one item per thread)
             const int m = e / per_row, j = e - m * per_row;
             *reinterpret_cast<u32x4*>(lds + m * kRowB + 16 * j) =
                 ld_agent_x4_wait(reinterpret_cast<const u32x4*>(p.act + (int64_t)m * (p.I / 4) + s0c * 8) + j);
@@ -227,8 +343,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
     __syncthreads();
     if (tid == 0) {
         const unsigned long long nd = (unsigned long long)p.GR * p.KC;
-        if (add_agent(p.sync + kWordStride * kWordDone, 1ull) == (launch + 1) * nd - 1)
+        if (add_agent(p.sync + kWordStride * kWordDone, 1ull) == (launch + 1) * nd - 1) {
             add_agent(p.sync + kWordStride * kWordLaunches, 1ull);
+            if (p.head > 0) add_agent(p.sync + kWordStride * kWordHeadLaunches, 1ull);
+        }
     }
 }
 
@@ -249,26 +367,30 @@ extern "C" int ksa_mlp_rows_down_splits(int H, int I) {
 }
 
 // Workspace: 32 KiB of counting words (to be zeroed once by the caller, and again after a launch
-// left the status word non-zero), then the activation [16][I] in 16-bit.
+// left the status word non-zero), then the activation [16][I] and the norm stage's rows [16][H] in 16-bit.
 extern "C" size_t ksa_mlp_rows_workspace_bytes(int H, int I) {
     if (H <= 0 || I <= 0) return 0;
-    return (size_t)kSyncWords * 8 + (size_t)16 * I * 2;
+    return (size_t)kSyncWords * 8 + (size_t)16 * I * 2 + (size_t)16 * H * 2;
 }
 
-extern "C" int ksa_mlp_rows(const void* x, const void* w_gate_up, const void* w_down, float* down_partials, int M,
-                            int H, int I, long long x_row_stride, long long w_gate_up_row_stride,
-                            long long w_down_row_stride, int dtype, void* workspace, size_t workspace_bytes,
-                            void* stream) {
-    if (!x || !w_gate_up || !w_down || !down_partials || !workspace) return KSA_ERR_NULL;
+namespace {
+
+// x given (head == 0) or made by the norm stage of the launch (x null)
+int mlp_rows_launch(const void* x, long long x_row_stride, const float* o_partials, int o_ksplit, const void* residual,
+                    const void* norm_weight, void* out_sum, long long residual_row_stride, long long sum_row_stride,
+                    float eps, const void* w_gate_up, const void* w_down, float* down_partials, int M, int H, int I,
+                    long long w_gate_up_row_stride, long long w_down_row_stride, int dtype, void* workspace,
+                    size_t workspace_bytes, void* stream) {
+    if (!w_gate_up || !w_down || !down_partials || !workspace) return KSA_ERR_NULL;
     if (M <= 0 || M > 16 || H <= 0 || I <= 0) return KSA_ERR_INVALID;
     if (H % 128 != 0 || I % 32 != 0) return KSA_ERR_UNSUPPORTED;  // four K slices of whole steps; whole steps of the down K
     if (dtype != KSA_DTYPE_BF16 && dtype != KSA_DTYPE_F16) return KSA_ERR_UNSUPPORTED;
     const int KC = ksa_mlp_rows_down_splits(H, I);
-    if (KC > kMaxChunks) return KSA_ERR_UNSUPPORTED;  // MLP sizes beyond 30720
+    if (KC > kMaxChunks) return KSA_ERR_UNSUPPORTED;  // MLP sizes beyond 26624
     if (workspace_bytes < ksa_mlp_rows_workspace_bytes(H, I)) return KSA_ERR_WORKSPACE;
     auto bad = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) != 0; };
-    if (bad(x) || bad(w_gate_up) || bad(w_down) || bad(down_partials) || bad(workspace)) return KSA_ERR_ALIGN;
-    if (x_row_stride % 8 || w_gate_up_row_stride % 8 || w_down_row_stride % 8) return KSA_ERR_ALIGN;
+    if (bad(w_gate_up) || bad(w_down) || bad(down_partials) || bad(workspace)) return KSA_ERR_ALIGN;
+    if (w_gate_up_row_stride % 8 || w_down_row_stride % 8) return KSA_ERR_ALIGN;
     const size_t lds = mlp_lds_bytes(M, H);
     if (lds > 160 * 1024) return KSA_ERR_UNSUPPORTED;
     auto kern = dtype == KSA_DTYPE_BF16 ? ksa_mlp_rows_kernel<KsaBf16> : ksa_mlp_rows_kernel<KsaF16>;
@@ -277,20 +399,64 @@ extern "C" int ksa_mlp_rows(const void* x, const void* w_gate_up, const void* w_
                             (int)lds) != hipSuccess)
         return KSA_ERR_LAUNCH;
     MlpParams p{};
-    p.x = (const uint16_t*)x;
     p.w_gu = (const uint16_t*)w_gate_up;
     p.w_dn = (const uint16_t*)w_down;
     p.dn_part = down_partials;
     p.sync = (unsigned long long*)workspace;
     p.act = p.sync + kSyncWords;
-    p.x_rs = x_row_stride, p.wgu_rs = w_gate_up_row_stride, p.wdn_rs = w_down_row_stride;
+    p.hbuf = p.act + (size_t)16 * I / 4;
+    p.wgu_rs = w_gate_up_row_stride, p.wdn_rs = w_down_row_stride;
     p.M = M, p.H = H, p.I = I;
     p.UB = I / 16;
     p.GR = (H / 16 + 2 * kSlices - 1) / (2 * kSlices);
     p.KC = KC;
     p.spin_limit = 1u << 19;  // polls of a microsecond or two: about a second
-    hipLaunchKernelGGL(kern, dim3(p.UB + p.GR * p.KC), dim3(128 * kSlices), lds, (hipStream_t)stream, p);
+    if (x) {
+        if (bad(x)) return KSA_ERR_ALIGN;
+        if (x_row_stride % 8) return KSA_ERR_ALIGN;
+        p.x = (const uint16_t*)x;
+        p.x_rs = x_row_stride;
+    } else {
+        if (!o_partials || !residual || !norm_weight || !out_sum) return KSA_ERR_NULL;
+        if (o_ksplit < 1 || o_ksplit > 64) return KSA_ERR_INVALID;
+        if (H > 4096) return KSA_ERR_UNSUPPORTED;  // a norm row is one 16-byte item per thread
+        if (bad(o_partials) || bad(residual) || bad(norm_weight) || bad(out_sum)) return KSA_ERR_ALIGN;
+        if (residual_row_stride % 8 || sum_row_stride % 8) return KSA_ERR_ALIGN;
+        p.o_part = o_partials;
+        p.o_ksplit = o_ksplit;
+        p.res = (const uint16_t*)residual;
+        p.norm_w = (const uint16_t*)norm_weight;
+        p.out_sum = (uint16_t*)out_sum;
+        p.res_rs = residual_row_stride, p.sum_rs = sum_row_stride;
+        p.eps = eps;
+        p.head = M;
+    }
+    hipLaunchKernelGGL(kern, dim3(p.head + p.UB + p.GR * p.KC), dim3(128 * kSlices), lds, (hipStream_t)stream, p);
     return ksa_check_launch();
+}
+
+}  // namespace
+
+extern "C" int ksa_mlp_rows(const void* x, const void* w_gate_up, const void* w_down, float* down_partials, int M,
+                            int H, int I, long long x_row_stride, long long w_gate_up_row_stride,
+                            long long w_down_row_stride, int dtype, void* workspace, size_t workspace_bytes,
+                            void* stream) {
+    if (!x) return KSA_ERR_NULL;
+    return mlp_rows_launch(x, x_row_stride, nullptr, 0, nullptr, nullptr, nullptr, 0, 0, 0.f, w_gate_up, w_down,
+                           down_partials, M, H, I, w_gate_up_row_stride, w_down_row_stride, dtype, workspace,
+                           workspace_bytes, stream);
+}
+
+extern "C" int ksa_add_rmsnorm_mlp_rows(const float* o_partials, int o_ksplit, const void* residual,
+                                        const void* norm_weight, void* out_sum, const void* w_gate_up,
+                                        const void* w_down, float* down_partials, int M, int H, int I,
+                                        long long residual_row_stride, long long sum_row_stride,
+                                        long long w_gate_up_row_stride, long long w_down_row_stride, int dtype,
+                                        float eps, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!o_partials) return KSA_ERR_NULL;
+    return mlp_rows_launch(nullptr, 0, o_partials, o_ksplit, residual, norm_weight, out_sum, residual_row_stride,
+                           sum_row_stride, eps, w_gate_up, w_down, down_partials, M, H, I, w_gate_up_row_stride,
+                           w_down_row_stride, dtype, workspace, workspace_bytes, stream);
 }
 
 // Status word of the workspace (device memory, 8 bytes at this offset): 0, or 1 after a launch in

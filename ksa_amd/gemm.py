@@ -101,7 +101,7 @@ class MlpRowsWorkspace:
 
 
 def mlp_rows_supported(M: int, H: int, I: int) -> bool:
-    return (1 <= M <= MAX_ROWS and H % 128 == 0 and I % 32 == 0 and I <= 30720
+    return (1 <= M <= MAX_ROWS and H % 128 == 0 and I % 32 == 0 and I <= 26624
             and M * (H + 8) * 2 <= 160 * 1024)
 
 
@@ -127,3 +127,32 @@ def mlp_rows(x: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor, ws:
                             ws.buf.numel(), _lib.stream_ptr(x2.device))
     _lib.check(rc, "ksa_mlp_rows")
     return SplitKPartials(part.view(torch.uint8), ks, M, x.shape, dt)
+
+
+def add_rmsnorm_mlp_rows(o_partials: SplitKPartials, residual: torch.Tensor, norm_weight: torch.Tensor, eps: float,
+                         w_gate_up: torch.Tensor, w_down: torch.Tensor, ws: MlpRowsWorkspace):
+    """One launch for `x' = residual + o_proj output; h = norm(x'); d = down(SiLU(gate(h)) * up(h))` at a
+    decode step (`ksa_add_rmsnorm_mlp_rows`; modeling_qwen3sa.py:944-952, :507-514).  Returns (x', d) with d
+    as `SplitKPartials` for the next residual add + norm."""
+    H = o_partials.shape[-1]
+    I = w_gate_up.shape[0] // 2
+    M = o_partials.rows
+    dt = o_partials.dtype
+    assert w_gate_up.shape == (2 * I, H) and w_down.shape == (H, I) and w_gate_up.dtype == dt and w_down.dtype == dt
+    assert w_gate_up.stride(1) == 1 and w_down.stride(1) == 1 and ws.H == H and ws.I == I and H <= 4096
+    r2 = residual.reshape(-1, H)
+    if r2.stride(1) != 1:
+        r2 = r2.contiguous()
+    assert r2.shape[0] == M and r2.dtype == dt
+    w = norm_weight.to(dt).contiguous()
+    L = _lib.lib()
+    with torch.cuda.device(r2.device):
+        ks = L.ksa_mlp_rows_down_splits(H, I)
+        out_sum = torch.empty(M, H, dtype=dt, device=r2.device)
+        part = torch.empty(ks * 16 * H, dtype=torch.float32, device=r2.device)
+        rc = L.ksa_add_rmsnorm_mlp_rows(o_partials.workspace.data_ptr(), o_partials.ksplit, r2.data_ptr(), w.data_ptr(),
+                                        out_sum.data_ptr(), w_gate_up.data_ptr(), w_down.data_ptr(), part.data_ptr(),
+                                        M, H, I, r2.stride(0), H, w_gate_up.stride(0), w_down.stride(0), _DT[dt],
+                                        float(eps), ws.buf.data_ptr(), ws.buf.numel(), _lib.stream_ptr(r2.device))
+    _lib.check(rc, "ksa_add_rmsnorm_mlp_rows")
+    return out_sum.view(residual.shape), SplitKPartials(part.view(torch.uint8), ks, M, residual.shape, dt)

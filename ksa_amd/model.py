@@ -174,6 +174,18 @@ class HipOps:
             return None
         return self._gemm.mlp_rows(x, w_gate_up, w_down, self.prepare_mlp_rows(H, I, x.device))
 
+    def add_norm_mlp_rows(self, o_partials, residual, norm_weight, eps, w_gate_up, w_down):
+        """(residual + o_proj output, down(SiLU(gate(h)) * up(h)) for h = norm of that sum) in one launch,
+        from the K-split partial sums of the o projection; None when the shapes are outside what the
+        kernel takes."""
+        if not isinstance(o_partials, self._gemm.SplitKPartials):
+            return None
+        H, I = residual.shape[-1], w_down.shape[1]
+        if not self._gemm.mlp_rows_supported(o_partials.rows, H, I) or H > 4096:
+            return None
+        return self._gemm.add_rmsnorm_mlp_rows(o_partials, residual, norm_weight, eps, w_gate_up, w_down,
+                                               self.prepare_mlp_rows(H, I, residual.device))
+
     def mlp_rows_failed(self):
         """True if a `mlp_rows` launch gave up waiting (synchronises); see `MlpRowsWorkspace.failed`."""
         return any(ws.failed() for ws in self._mlp_ws.values())
@@ -286,6 +298,18 @@ class KsaQwen3ForCausalLM:
         if delta is None:
             return self.ops.add_rmsnorm(x, None, w, self.config.rms_norm_eps)
         return self.ops.add_rmsnorm(delta, x, w, self.config.rms_norm_eps)
+
+    def _post_attention(self, lw, attn, x):
+        """The second half of a layer at a decode step, from the attention output: (x', delta) with
+        x' = x + o_proj(attn) and delta = mlp(post_attention_layernorm(x')) (deferred sums)."""
+        o = self.ops.linear(attn, lw["o_proj"], defer=True)
+        if hasattr(self.ops, "add_norm_mlp_rows"):
+            out = self.ops.add_norm_mlp_rows(o, x, lw["post_attention_layernorm"], self.config.rms_norm_eps,
+                                             lw["gate_up_proj"], lw["down_proj"])
+            if out is not None:
+                return out
+        x, h = self._add_norm(o, x, lw["post_attention_layernorm"])
+        return x, self._mlp(lw, h, defer=True)
 
     def _rope_tables(self, position_ids):
         """cos, sin [1, L, D] in the model dtype from position ids [1, L] (computed in fp32)."""
@@ -426,9 +450,12 @@ class KsaQwen3ForCausalLM:
                 cache.update_summary(kh[:, :, 1:], vh[:, :, 1:], li)
                 attn = torch.cat([text_out, sum_out], dim=1)
             # a text step hands both products straight to the next norm; a boundary step slices them
-            x, h = self._add_norm(ops.linear(attn.reshape(b, ids.shape[1], -1), lw["o_proj"], defer=not boundary),
-                                  x, lw["post_attention_layernorm"])
-            delta = self._mlp(lw, h, defer=not boundary)
+            if boundary:
+                x, h = self._add_norm(ops.linear(attn.reshape(b, ids.shape[1], -1), lw["o_proj"]), x,
+                                      lw["post_attention_layernorm"])
+                delta = self._mlp(lw, h)
+            else:
+                x, delta = self._post_attention(lw, attn.reshape(b, ids.shape[1], -1), x)
         cache.reset_chunk_counter()
         if not boundary:
             return self._logits(x, delta)
@@ -461,9 +488,7 @@ class KsaQwen3ForCausalLM:
                                                      cfg.rms_norm_eps, **slots)
             attn = ops.decode(q.transpose(1, 2), cache.key_cache[li], cache.value_cache[li],
                               st["cur"][kind, 1], st["cur"][kind, 2], self.scaling)
-            x, h = self._add_norm(ops.linear(attn.reshape(b, 1, -1), lw["o_proj"], defer=True), x,
-                                  lw["post_attention_layernorm"])
-            delta = self._mlp(lw, h, defer=True)
+            x, delta = self._post_attention(lw, attn.reshape(b, 1, -1), x)
         return self._logits(x, delta)
 
     @torch.no_grad()

@@ -163,3 +163,42 @@ def test_gpu_mlp_rows_one_launch(dtype, M, H, I):
         ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
         diff = (d_new.float() - d_ref[0].float()).abs()
         assert (diff <= 2 * ulp * d_ref[0].float().abs() + 4 * ulp * want.abs().max().item() * 2.0 ** -6).all(), diff.max()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,H,I", [(8, 2560, 9728), (1, 2560, 9728), (16, 1024, 768), (3, 128, 64), (5, 4096, 512)])
+def test_gpu_add_rmsnorm_mlp_rows_one_launch(dtype, M, H, I):
+    """Residual add + norm + MLP in one launch against ksa_add_rmsnorm_partials followed by ksa_mlp_rows:
+    the sum with the residual bit-identical; the down projection (added up from its partial sums) to
+    within what a last-place difference of a few normalised values can move it.  Three launches on one
+    workspace, mixed with launches of the form without the norm stage."""
+    from ksa_amd import add_rmsnorm
+    from ksa_amd.gemm import MlpRowsWorkspace, SplitKPartials, add_rmsnorm_mlp_rows, linear_rows, mlp_rows
+    g = torch.Generator().manual_seed(M * 7 + H + I)
+    dev = torch.device("cuda")
+    Ko = 512 if H <= 1024 else 4096
+    attn = torch.randn(1, M, Ko, generator=g).to(dtype).to(dev)
+    w_o = (torch.randn(H, Ko, generator=g) * 0.03).to(dtype).to(dev)
+    res = torch.randn(1, M, H, generator=g).to(dtype).to(dev)
+    nw = (1 + 0.1 * torch.randn(H, generator=g)).to(dtype).to(dev)
+    w_gu = (torch.randn(2 * I, H, generator=g) * 0.04).to(dtype).to(dev)
+    w_dn = (torch.randn(H, I, generator=g) * 0.03).to(dtype).to(dev)
+    o = linear_rows(attn, w_o, defer=True)
+    if not isinstance(o, SplitKPartials):  # K too short to be split: present the product as one slice
+        ws1 = torch.zeros(16, H, dtype=torch.float32, device=dev)
+        ws1[:M] = o[0].float()
+        o = SplitKPartials(ws1.view(-1).view(torch.uint8), 1, M, (1, M, H), dtype)
+    ws = MlpRowsWorkspace(H, I, dev)
+    x_ref, h_ref = add_rmsnorm(o, res, nw, 1e-6)
+    d_ref = mlp_rows(h_ref, w_gu, w_dn, ws)
+    sum_ref = d_ref.workspace.view(torch.float32).view(d_ref.ksplit, 16, H)[:, :M].sum(0)
+    for rep in range(3):
+        x_new, d_new = add_rmsnorm_mlp_rows(o, res, nw, 1e-6, w_gu, w_dn, ws)
+        torch.cuda.synchronize()
+        assert not ws.failed(), "a workgroup gave up waiting"
+        assert torch.equal(x_new, x_ref)
+        sum_new = d_new.workspace.view(torch.float32).view(d_new.ksplit, 16, H)[:, :M].sum(0)
+        assert (sum_new - sum_ref).abs().max().item() <= 4e-3 * sum_ref.abs().max().item() + 1e-5
+        if rep == 1:
+            mlp_rows(h_ref, w_gu, w_dn, ws)
