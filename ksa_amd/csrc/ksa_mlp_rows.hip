@@ -43,6 +43,7 @@
 namespace {
 
 constexpr int kSlices = 4;        // K slices of the hidden size = waves per gate / up half
+constexpr int kTileCols = 16;     // columns of the activation per gate | up workgroup (8: same time, twice the reads of x)
 constexpr int kWordStride = 64;   // 64-bit words are 512 bytes apart
 // words: [0] launches so far, [1] down workgroups done, [2] status, [4 .. 11] rows of the norm stage done
 // (eight copies, a gate | up workgroup watches copy number % 8: hundreds of workgroups polling one
@@ -173,17 +174,21 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
     }
     const int bid = blockIdx.x - p.head;  // number among the workgroups of the two products
     if (bid < p.UB) {
-        // ---- 16 columns of the activation (ksa_gemm_gate_up_silu_kernel's scheme) ----
+        // ---- kTileCols columns of the activation (ksa_gemm_gate_up_silu_kernel's scheme; with fewer than
+        // 16 columns the rows of W beyond them are not requested) ----
         const int u = bid;
         const int half = wave / kSlices;  // 0: gate rows of w, 1: up rows
         const int slice = wave - half * kSlices;
         const int sl_steps = p.H / 32 / kSlices;  // K steps of a slice (H is a multiple of 128)
         const int rowb = (p.H + 8) * 2;
-        const uint16_t* wp = p.w_gu + ((int64_t)half * p.I + min(16 * u + r, p.I - 1)) * p.wgu_rs +
+        const uint16_t* wp = p.w_gu + ((int64_t)half * p.I + min(kTileCols * u + (r & (kTileCols - 1)), p.I - 1)) * p.wgu_rs +
                              32 * (slice * sl_steps) + 8 * kq;
         auto load_steps = [&](int s0) {  // (steps beyond the slice repeat its last one and are not multiplied)
+            if (r < kTileCols) {
 #pragma unroll
-            for (int k = 0; k < kB; ++k) a[k] = *reinterpret_cast<const u32x4*>(wp + 32 * min(s0 + k, sl_steps - 1));
+                for (int k = 0; k < kB; ++k)
+                    a[k] = *reinterpret_cast<const u32x4*>(wp + 32 * min(s0 + k, sl_steps - 1));
+            }
         };
         load_steps(0);  // in flight while x is waited for and staged
         if (p.head > 0) {
@@ -241,8 +246,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
         for (int i = 0; i < 4; ++i) red[(wave * 16 + r) * 17 + 4 * kq + i] = acc[i];
         __syncthreads();
         if (tid < 64) {  // (row m, four columns): the slices added in order, SiLU, product; one 8-byte store
-            const int m = tid >> 2, c0 = 4 * (tid & 3);
-            if (m < p.M && 16 * u + c0 < p.I) {
+            constexpr int kQuads = kTileCols / 4;
+            const int m = tid / kQuads, c0 = 4 * (tid % kQuads);
+            if (m < p.M && m < 16 && kTileCols * u + c0 < p.I) {
                 unsigned long long o = 0;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
@@ -256,11 +262,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
                     const float sl_ = C::up(C::down(gs / (1.f + expf(-gs))));
                     o |= (unsigned long long)C::down(sl_ * us) << (16 * e);
                 }
-                st_agent(p.act + (int64_t)m * (p.I / 4) + 4 * u + (tid & 3), o);
+                st_agent(p.act + (int64_t)m * (p.I / 4) + kQuads * u + (tid % kQuads), o);
             }
             // the stores are complete (this wave made all of them) before the tile is counted off
             __builtin_amdgcn_s_waitcnt(0);
-            if (tid == 0) add_agent(p.sync + kWordStride * (kWordChunk0 + u / 32), 1ull);
+            if (tid == 0) add_agent(p.sync + kWordStride * (kWordChunk0 + u / (kChunkK / kTileCols)), 1ull);
         }
         return;
     }
@@ -288,7 +294,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
         launch = ld_agent(p.sync + kWordStride * kWordLaunches);
         launch = (unsigned long long)__builtin_amdgcn_readfirstlane((unsigned)launch) |  // (kept in scalar registers)
                  ((unsigned long long)__builtin_amdgcn_readfirstlane((unsigned)(launch >> 32)) << 32);
-        const int tiles = min(32, p.UB - 32 * kc);
+        const int tiles = min(kChunkK / kTileCols, p.UB - (kChunkK / kTileCols) * kc);
         const unsigned long long want = (launch + 1) * (unsigned long long)tiles;
         unsigned long long* word = p.sync + kWordStride * (kWordChunk0 + kc);
         unsigned long long* status = p.sync + kWordStride * kWordStatus;
@@ -407,7 +413,7 @@ int mlp_rows_launch(const void* x, long long x_row_stride, const float* o_partia
     p.hbuf = p.act + (size_t)16 * I / 4;
     p.wgu_rs = w_gate_up_row_stride, p.wdn_rs = w_down_row_stride;
     p.M = M, p.H = H, p.I = I;
-    p.UB = I / 16;
+    p.UB = I / kTileCols;
     p.GR = (H / 16 + 2 * kSlices - 1) / (2 * kSlices);
     p.KC = KC;
     p.spin_limit = 1u << 19;  // polls of a microsecond or two: about a second
