@@ -9,7 +9,8 @@
  * Conventions
  *   - every pointer is a DEVICE pointer owned by the caller unless stated otherwise;
  *     the library never allocates, frees or synchronises, keeps no state between calls (the one
- *     exception, a fixed scratch array, is described at ksa_decode_fwd_noalloc) and reads no
+ *     exception, a fixed scratch array, is described at ksa_decode_fwd_noalloc; ksa_mlp_rows keeps
+ *     counting words in a workspace that the caller owns and zeroes once) and reads no
  *     environment variable;
  *   - `stream` is a hipStream_t passed as void* (0 = the null stream);
  *   - 16-bit tensors are described by element strides; pointers must be 16-byte
