@@ -127,7 +127,7 @@ def test_gpu_gate_up_silu_one_launch(dtype, M, I, K):
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("M,H,I", [(8, 2560, 9728), (1, 2560, 9728), (16, 1024, 768), (3, 256, 256), (5, 4096, 512),
-                                   (8, 768, 2304)])
+                                   (8, 768, 2304), (16, 2560, 1024)])
 def test_gpu_mlp_rows_one_launch(dtype, M, H, I):
     """The MLP of a layer in one launch of resident workgroups (gate | up + SiLU -> grid barrier ->
     down) against the two separate launches it stands for: the down projection, added up from its
@@ -167,7 +167,8 @@ def test_gpu_mlp_rows_one_launch(dtype, M, H, I):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("M,H,I", [(8, 2560, 9728), (1, 2560, 9728), (16, 1024, 768), (3, 128, 64), (5, 4096, 512)])
+@pytest.mark.parametrize("M,H,I", [(8, 2560, 9728), (1, 2560, 9728), (16, 1024, 768), (3, 128, 64), (5, 4096, 512),
+                                   (16, 2560, 1024)])
 def test_gpu_add_rmsnorm_mlp_rows_one_launch(dtype, M, H, I):
     """Residual add + norm + MLP in one launch against ksa_add_rmsnorm_partials followed by ksa_mlp_rows:
     the sum with the residual bit-identical; the down projection (added up from its partial sums) to
