@@ -563,11 +563,19 @@ class KsaQwen3ForCausalLM:
         st["rope_rel"].fill_(p - st["rope_p0"])
         ptrs = tuple((t.data_ptr(), tuple(t.shape), t.stride()) for t in cache.key_cache + cache.value_cache)
         if st["graph"] is None or st["ptrs"] != ptrs:
-            side = torch.cuda.Stream(device=self.device)
-            side.wait_stream(torch.cuda.current_stream(self.device))
-            with torch.cuda.stream(side):   # the step is idempotent: run it once before recording it
-                self._text_step_body(st, cache)
-            torch.cuda.current_stream(self.device).wait_stream(side)
+            warm = getattr(self, "_graph_warm", None)
+            if warm is None:
+                warm = self._graph_warm = set()
+            if b not in warm:
+                # The step is idempotent: the first recording for a batch size runs it once on a side
+                # stream beforehand, so that everything that happens lazily (kernel modules, workspaces)
+                # happens outside the capture.  Later recordings (a new cache) need no such run.
+                side = torch.cuda.Stream(device=self.device)
+                side.wait_stream(torch.cuda.current_stream(self.device))
+                with torch.cuda.stream(side):
+                    self._text_step_body(st, cache)
+                torch.cuda.current_stream(self.device).wait_stream(side)
+                warm.add(b)
             g = torch.cuda.CUDAGraph()
             with torch.cuda.graph(g):
                 st["logits"] = self._text_step_body(st, cache)
