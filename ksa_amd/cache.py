@@ -272,6 +272,58 @@ class Qwen3RingBufferCache:
         self.cur_chunk_sizes[layer_idx] += n_new
         self._total_chunks[layer_idx] += n_new
 
+    def boundary_fits_one_piece(self, layer_idx: int) -> bool:
+        """True when the flush of a chunk-boundary step that starts now (the chunk's last text row
+        still to come) is one run of rows in the ring, i.e. `boundary_slots` can describe it."""
+        if self.is_large_window[layer_idx]:
+            return True
+        cbl = self._chunk_buf_len[layer_idx] + 1
+        return cbl <= self.window_sizes[layer_idx] - self._window_write_ptr[layer_idx]
+
+    def boundary_slots(self, layer_idx: int, n_new: int):
+        """`update_text` of a chunk's last text token followed by `update_summary` of its `n_new`
+        summary rows, without moving a row: advances the counters (enlarging a buffer that is too
+        small) and returns the rows the two calls would have used, for a caller that moves the
+        rows itself (a launch sequence replayed with the rows in device memory):
+
+            small window: text (row of the text token), attend (start, end of the text query's
+                          range, taken between the two calls as `decode_step` does), flush_src,
+                          flush_dst, flush_rows (chunk rows -> ring), append (row of the first
+                          new summary)
+            large window: text, attend, and spare = the first of `n_new` rows behind the text that
+                          the caller may use for the summary rows of the step (they are not kept)
+
+        Requires `boundary_fits_one_piece(layer_idx)`."""
+        C, S = self.summary_chunk_size, self.summary_token_num
+        if self.is_large_window[layer_idx]:
+            row = self._text_len[layer_idx]
+            if row + 1 + n_new > self._capacity[layer_idx]:
+                self._regrow(layer_idx, max(row + 1 + n_new + self._APPEND_HEADROOM,
+                                            2 * self._capacity[layer_idx]), row)
+            self._text_len[layer_idx] = row + 1
+            out = dict(text=row, attend=(0, row + 1), spare=row + 1)
+        else:
+            assert self.boundary_fits_one_piece(layer_idx)
+            ws = self.window_sizes[layer_idx]
+            cbl = self._chunk_buf_len[layer_idx] + 1
+            row = S + C - cbl
+            self._chunk_buf_len[layer_idx] = cbl
+            attend = self.attention_range(layer_idx)
+            ptr = self._window_write_ptr[layer_idx]
+            self._window_write_ptr[layer_idx] = (ptr + cbl) % ws
+            self._n_valid_window[layer_idx] = min(ws, self._n_valid_window[layer_idx] + cbl)
+            self._chunk_buf_len[layer_idx] = 0
+            dst = S + C + ws + self._n_summaries[layer_idx]
+            if dst + n_new > self._capacity[layer_idx]:
+                self._grow_buffer_right(layer_idx)
+            self._n_summaries[layer_idx] += n_new
+            out = dict(text=row, attend=attend, flush_src=row, flush_dst=S + C + ptr, flush_rows=cbl,
+                       append=dst)
+        self.cur_chunk_sizes[layer_idx] += 1 + n_new
+        self.true_tokens[layer_idx] += 1
+        self._total_chunks[layer_idx] += n_new
+        return out
+
     def attention_range(self, layer_idx: int):
         """Row range [start, end) a text query attends (the slice of get_attention_kv)."""
         if self.is_large_window[layer_idx]:

@@ -275,6 +275,12 @@ class KsaQwen3ForCausalLM:
     """Inference-only decoder: `forward` for one prefill or one decode step, `generate` for a
     greedy loop.  All sequences of a batch have the same length."""
 
+    # `decode_step_graph` runs this many chunk-boundary steps of a cache eagerly before it records
+    # them: recording the roughly 800 launches of a boundary step costs about as much host time as
+    # three eager boundary steps lose against replayed ones, so a short generation never pays for a
+    # recording it does not use, and a long one pays at most twice the best possible.
+    BOUNDARY_GRAPH_AFTER = 3
+
     def __init__(self, config: KsaQwen3Config, weights: dict, ops=None):
         self.config = config
         self.w = weights
@@ -491,61 +497,181 @@ class KsaQwen3ForCausalLM:
             x, delta = self._post_attention(lw, attn.reshape(b, 1, -1), x)
         return self._logits(x, delta)
 
+    def _boundary_step_body(self, st, cache):
+        """One chunk-boundary decode step in the recordable form of `_text_step_body`: the text
+        token and the chunk's S summary tokens run together, and every row that `decode_step` takes
+        from the cache's counters (where the text row goes, the text query's range, where the chunk
+        is flushed to in the ring, where the new summaries are appended) is read from `st["bcur"]`:
+
+            [0: small window][text row, range start, range end, flush destination, append row, -]
+            [1: large window][text row, range start, range end, first spare row behind the text,
+                              start and end of [chunk text | spare rows]]
+
+        In a large-window layer the summary rows' K/V sit in spare rows behind the text for the
+        length of the step (the next text token overwrites them), which gives the summary queries
+        the [chunk | own summaries] rows of `get_summary_attention_kv` as one row range."""
+        cfg, ops = self.config, self.ops
+        C, S = cfg.summary_chunk_size, cfg.summary_token_num
+        ids, bc = st["btok"], st["bcur"]
+        b = ids.shape[0]
+        sum_rows = st["bsum_rows"]
+        cos, sin = self._rope_tables(st["bpos"])
+        x = self.w["embed_tokens"][ids]
+        delta = None
+        for li, lw in enumerate(self.w["layers"]):
+            kind = 1 if cache.is_large_window[li] else 0
+            kc, vc, mv = cache.key_cache[li], cache.value_cache[li], cache._move_rows
+            x, h = self._add_norm(delta, x, lw["input_layernorm"])
+            q, k, v = self._qkv(lw, h, sum_rows)
+            q, k, v = ops.pre_attention(q, k, v, lw["q_norm"], lw["k_norm"], cos, sin, cfg.rms_norm_eps)
+            self._blend_summary(lw, h, sum_rows, cos, sin, q, k, v)
+            qh, kh, vh = q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2)
+            mv(kh[:, :, :1], kc, 1, dst_start_seq=bc[kind, 0])
+            mv(vh[:, :, :1], vc, 1, dst_start_seq=bc[kind, 0])
+            text_out = ops.decode(qh[:, :, :1], kc, vc, bc[kind, 1], bc[kind, 2], self.scaling)
+            if kind == 0:
+                mv(kh[:, :, 1:], kc, S, 0, 0)
+                mv(vh[:, :, 1:], vc, S, 0, 0)
+                sum_out = ops.decode(qh[:, :, 1:], kc[:, :, :S + C], vc[:, :, :S + C], 0, S + C, self.scaling)
+                for buf, new in ((kc, kh), (vc, vh)):
+                    mv(buf, buf, C, S, dst_start_seq=bc[0, 3])            # chunk rows -> ring
+                    mv(new[:, :, 1:], buf, S, dst_start_seq=bc[0, 4])     # the chunk's summaries
+            else:
+                mv(kh[:, :, 1:], kc, S, dst_start_seq=bc[1, 3])
+                mv(vh[:, :, 1:], vc, S, dst_start_seq=bc[1, 3])
+                sum_out = ops.decode(qh[:, :, 1:], kc, vc, bc[1, 4], bc[1, 5], self.scaling)
+            attn = torch.cat([text_out, sum_out], dim=1)
+            x, h = self._add_norm(ops.linear(attn.reshape(b, 1 + S, -1), lw["o_proj"]), x,
+                                  lw["post_attention_layernorm"])
+            delta = self._mlp(lw, h)
+        return self._logits(x[:, :1], delta[:, :1])
+
+    def _stage_ints(self, st, key, vals):
+        """Host integers `vals` (a flat list) -> the int32 device tensor st[key], through a ring of
+        pinned host slots: a copy from pageable memory would hold the host until the GPU has reached
+        it, i.e. until the previous step has ended, and the GPU would then idle while the host
+        prepares the next replay.  A slot is written again only after the copy that read it has run
+        (its event), so the host may be up to a ring's length of steps ahead of the GPU."""
+        ring = st["rings"].get(key)
+        if ring is None:
+            ring = st["rings"][key] = {"slots": torch.empty(16, len(vals), dtype=torch.int32, pin_memory=True),
+                                       "events": [None] * 16, "next": 0}
+        slot = ring["next"]
+        ring["next"] = (slot + 1) % 16
+        if ring["events"][slot] is not None:
+            ring["events"][slot].synchronize()
+        ring["slots"][slot].copy_(torch.tensor(vals, dtype=torch.int32))
+        st[key].view(-1).copy_(ring["slots"][slot], non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record(torch.cuda.current_stream(self.device))
+        ring["events"][slot] = ev
+
+    def _warm_up(self, st, which, body, cache):
+        """Runs `body` once, launched eagerly on a side stream, the first time a recording of this
+        kind is needed for a batch size, so that everything that happens lazily (kernel modules,
+        GEMM handles, workspaces) happens outside the capture.  Returns whether it ran."""
+        warm = getattr(self, "_graph_warm", None)
+        if warm is None:
+            warm = self._graph_warm = set()
+        if (which, st["batch"]) in warm:
+            return False
+        side = torch.cuda.Stream(device=self.device)
+        side.wait_stream(torch.cuda.current_stream(self.device))
+        with torch.cuda.stream(side):
+            body(st, cache)
+        torch.cuda.current_stream(self.device).wait_stream(side)
+        warm.add((which, st["batch"]))
+        return True
+
+    def _replay(self, st, which, body, cache):
+        """Replays the recording `which` of `body`, recording it first when there is none for the
+        cache buffers as they are now (the launches bake in addresses, strides and capacity)."""
+        ptrs = tuple((t.data_ptr(), tuple(t.shape), t.stride()) for t in cache.key_cache + cache.value_cache)
+        rec = st["graphs"].get(which)
+        if rec is None or rec["ptrs"] != ptrs:
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                logits = body(st, cache)
+            rec = st["graphs"][which] = {"graph": g, "ptrs": ptrs, "logits": logits}
+        rec["graph"].replay()
+        return rec["logits"]
+
     @torch.no_grad()
     def decode_step_graph(self, token_ids: torch.Tensor, cache):
-        """`decode_step` with the launches of a non-boundary step replayed from a HIP graph (about
-        400 launches per step otherwise cost more host time than GPU time).  Chunk-boundary steps
-        run as in `decode_step`.  The recording belongs to the cache object it was made for (it is
-        kept on it) and is made again when a cache buffer was reallocated or changed its shape:
-        the launches bake in the buffers' addresses, strides and capacity.
-        The returned logits live in a buffer that the next call overwrites."""
+        """`decode_step` with the launches of a step replayed from a HIP graph (about 400 launches
+        per step otherwise cost more host time than GPU time): one recording for the steps inside a
+        chunk, one for the chunk-boundary steps.  The recordings belong to the cache object they
+        were made for (they are kept on it) and are made again when a cache buffer was reallocated
+        or changed its shape.  The returned logits live in a buffer that a later call overwrites."""
         cfg = self.config
         C, S = cfg.summary_chunk_size, cfg.summary_token_num
-        if cache.get_cur_chunk_size() == C - 1:
-            return self.decode_step(token_ids, cache)
         b = token_ids.shape[0]
         Hkv, D = cfg.num_key_value_heads, cfg.head_dim
+        nl = cfg.num_hidden_layers
         st = getattr(cache, "_ksa_graph_state", None)
         if st is None or st["batch"] != b or st["owner"] is not self:
-            st = {"batch": b, "owner": self, "graph": None, "ptrs": None,
+            sids = torch.arange(S, device=self.device, dtype=torch.long) + cfg.summary_token_begin
+            st = {"batch": b, "owner": self, "graphs": {}, "rings": {},
                   "tok": torch.zeros(b, 1, dtype=torch.long, device=self.device),
                   # [kind: small / large window][destination row, range start, range end][sequence]
-                  "cur": torch.zeros(2, 3, b, dtype=torch.int32, device=self.device)}
+                  "cur": torch.zeros(2, 3, b, dtype=torch.int32, device=self.device),
+                  # the same for a boundary step (see `_boundary_step_body`), its ids and positions
+                  "bcur": torch.zeros(2, 6, b, dtype=torch.int32, device=self.device),
+                  "btok": torch.cat([torch.zeros(b, 1, dtype=torch.long, device=self.device),
+                                     sids[None].expand(b, -1)], dim=1).contiguous(),
+                  "bpos": torch.zeros(1, 1 + S, dtype=torch.int32, device=self.device),
+                  "bsum_rows": torch.arange(1, 1 + S, device=self.device)}
             cache._ksa_graph_state = st
+        kinds = [1 if cache.is_large_window[li] else 0 for li in range(nl)]
+        if cache.get_cur_chunk_size() == C - 1:
+            # recorded: a boundary step whose flush is one whole chunk in one piece (every boundary of
+            # a cache filled by `prefill`), once the cache has seen enough of them; else eagerly
+            st["boundaries"] = st.get("boundaries", 0) + 1
+            if st["boundaries"] <= self.BOUNDARY_GRAPH_AFTER or not all(
+                    cache.boundary_fits_one_piece(li) and (kinds[li] or cache._chunk_buf_len[li] == C - 1)
+                    for li in range(nl)):
+                return self.decode_step(token_ids, cache)
+            pos = boundary_position_ids(cache.get_true_token_num(), cfg, "cpu")[0].tolist()
+            vals = [[0, 0, 1, 0, 0, 0], [0, 0, 1, 0, 0, 1]]
+            seen = [None, None]
+            for li in range(nl):
+                sl = cache.boundary_slots(li, S)
+                a, e = sl["attend"]
+                if kinds[li]:
+                    row = [sl["text"], a, e, sl["spare"], sl["spare"] - C, sl["spare"] + S]
+                else:
+                    assert sl["flush_src"] == S and sl["flush_rows"] == C
+                    row = [sl["text"], a, e, sl["flush_dst"], sl["append"], 0]
+                assert seen[kinds[li]] in (None, row), "layers of one kind must move in step"
+                seen[kinds[li]] = vals[kinds[li]] = row
+            self._stage_ints(st, "bpos", pos)
+            st["btok"][:, :1].copy_(token_ids.to(self.device))
+            # A boundary step is not idempotent (its flush overwrites ring rows that its text query
+            # still attends), so the warm-up run flushes the chunk onto itself and appends the
+            # summaries onto the scratch rows that already hold them.
+            if ("boundary", b) not in getattr(self, "_graph_warm", ()):
+                harmless = [vals[0][:3] + [S, 0, 0], vals[1]]
+                self._stage_ints(st, "bcur", [v for kind in harmless for x in kind for v in [x] * b])
+                self._warm_up(st, "boundary", self._boundary_step_body, cache)
+            self._stage_ints(st, "bcur", [v for kind in vals for x in kind for v in [x] * b])
+            logits = self._replay(st, "boundary", self._boundary_step_body, cache)
+            cache.reset_chunk_counter()
+            return logits
         p = cache.get_true_token_num() if cfg.summary_chunk_position_ids_type == "origin" \
             else cache.get_cur_chunk_size()
         # host bookkeeping of the step (may enlarge an append-only buffer), then this step's rows
         rows = [None, None]
-        for li in range(cfg.num_hidden_layers):
-            kind = 1 if cache.is_large_window[li] else 0
-            if rows[kind] is None:
-                rows[kind] = cache._text_len[li] if kind else S + C - 1 - cache._chunk_buf_len[li]
+        for li in range(nl):
+            if rows[kinds[li]] is None:
+                rows[kinds[li]] = cache._text_len[li] if kinds[li] else S + C - 1 - cache._chunk_buf_len[li]
             cache.text_slots(li, b, Hkv, D, self.dtype, self.device)
         vals = [[0, 0, 1], [0, 0, 1]]
-        for li in range(cfg.num_hidden_layers):
-            kind = 1 if cache.is_large_window[li] else 0
-            if rows[kind] is not None:
+        for li in range(nl):
+            if rows[kinds[li]] is not None:
                 a, e = cache.attention_range(li)
-                vals[kind] = [rows[kind], a, e]
-                rows[kind] = None
-        # The values travel through a ring of pinned host slots: a copy from pageable memory would
-        # hold the host until the GPU has reached it, i.e. until the previous step has ended, and
-        # the GPU would then idle while the host prepares the next replay.  A slot is written again
-        # only after the copy that read it has run (its event), so the host may be up to a ring's
-        # length of steps ahead of the GPU.
-        if "ring" not in st:
-            st["ring"] = torch.empty(16, 2, 3, b, dtype=torch.int32, pin_memory=True)
-            st["ring_events"] = [None] * 16
-            st["ring_next"] = 0
-        slot = st["ring_next"]
-        st["ring_next"] = (slot + 1) % 16
-        if st["ring_events"][slot] is not None:
-            st["ring_events"][slot].synchronize()
-        st["ring"][slot].copy_(torch.tensor(vals, dtype=torch.int32).view(2, 3, 1))
-        st["cur"].copy_(st["ring"][slot], non_blocking=True)
-        ev = torch.cuda.Event()
-        ev.record(torch.cuda.current_stream(self.device))
-        st["ring_events"][slot] = ev
+                vals[kinds[li]] = [rows[kinds[li]], a, e]
+                rows[kinds[li]] = None
+        self._stage_ints(st, "cur", [v for kind in vals for x in kind for v in [x] * b])
         st["tok"].copy_(token_ids.to(self.device))
         # rotary rows of a window of positions, made with the prefill's own tensor ops (so a step's
         # cos / sin are the values `_rope_tables` gives) and refilled in place when p leaves it; the
@@ -561,28 +687,10 @@ class KsaQwen3ForCausalLM:
                 st["rope_rel"] = torch.zeros(1, dtype=torch.long, device=self.device)
             st["rope_p0"] = p
         st["rope_rel"].fill_(p - st["rope_p0"])
-        ptrs = tuple((t.data_ptr(), tuple(t.shape), t.stride()) for t in cache.key_cache + cache.value_cache)
-        if st["graph"] is None or st["ptrs"] != ptrs:
-            warm = getattr(self, "_graph_warm", None)
-            if warm is None:
-                warm = self._graph_warm = set()
-            if b not in warm:
-                # The step is idempotent: the first recording for a batch size runs it once on a side
-                # stream beforehand, so that everything that happens lazily (kernel modules, workspaces)
-                # happens outside the capture.  Later recordings (a new cache) need no such run.
-                side = torch.cuda.Stream(device=self.device)
-                side.wait_stream(torch.cuda.current_stream(self.device))
-                with torch.cuda.stream(side):
-                    self._text_step_body(st, cache)
-                torch.cuda.current_stream(self.device).wait_stream(side)
-                warm.add(b)
-            g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g):
-                st["logits"] = self._text_step_body(st, cache)
-            st["graph"], st["ptrs"] = g, ptrs
-        st["graph"].replay()
+        self._warm_up(st, "text", self._text_step_body, cache)   # a step inside a chunk is idempotent
+        logits = self._replay(st, "text", self._text_step_body, cache)
         cache.reset_chunk_counter()
-        return st["logits"]
+        return logits
 
     # ---- driver ----------------------------------------------------------------------
     def forward(self, input_ids: torch.Tensor, cache=None):
@@ -597,7 +705,7 @@ class KsaQwen3ForCausalLM:
         """Greedy decoding.  Returns ids [b, n + max_new_tokens] (and the logits of every step,
         [b, max_new_tokens, vocab], on request).  `forced` [b, max_new_tokens] replaces the
         arg-max token fed back at every step (teacher forcing, for comparing two runs).
-        `use_graph` replays the non-boundary decode steps from a HIP graph."""
+        `use_graph` replays the decode steps from HIP graphs (`decode_step_graph`)."""
         logits, cache = self.prefill(input_ids)
         out, steps = [], []
         for t in range(max_new_tokens):

@@ -154,6 +154,79 @@ def test_cache_bookkeeping_matches_model(C, S, n_prefill):
             check()
 
 
+@pytest.mark.parametrize("C,S,n_prefill", [(4, 2, 7), (8, 1, 16), (4, 2, 1), (2, 1, 3)])
+def test_cache_boundary_slots_equal_update_calls(C, S, n_prefill):
+    """`boundary_slots` + the caller's own row moves (what the recorded boundary step does)
+    against `update_text` + `get_summary_attention_kv` + `update_summary` on a second cache
+    driven with the same rows: same counters, same ranges, same buffer contents wherever
+    rows are attended, over many boundaries (ring wrap-around, growth of the summary region)."""
+    scns = [2, 3, 1000]
+    a_cache, b_cache = _make_cache(C, S, scns), _make_cache(C, S, scns)
+    for c in (a_cache, b_cache):
+        c._SUMMARY_INIT_CAP = 4
+        c._APPEND_HEADROOM = 5
+    B = C + S
+    Sq = (n_prefill // C) * B + n_prefill % C
+    sp = torch.from_numpy(O.summary_positions(Sq, C, S))[None]
+    D, H = 8, 2
+    kv = torch.arange(Sq, dtype=torch.float32)[None, None, :, None].expand(1, H, Sq, D).to(torch.bfloat16).contiguous()
+    for c in (a_cache, b_cache):
+        for layer in range(3):
+            c.update(kv, kv, layer, {"summary_mask": sp})
+        c.reorganize_after_prefill(sp)
+    pos, n_text, n_boundaries = Sq, n_prefill, 0
+    counters = ("_text_len", "_capacity", "_window_write_ptr", "_n_valid_window", "_chunk_buf_len",
+                "_n_summaries", "cur_chunk_sizes", "true_tokens", "_total_chunks")
+    for _ in range(40 * C):
+        row = torch.full((1, H, 1, D), float(pos % 251), dtype=torch.bfloat16)
+        boundary = n_text % C == C - 1
+        if not boundary:
+            for layer in range(3):
+                a_cache.update_text(row, row, layer)
+                b_cache.update_text(row, row, layer)
+            pos += 1
+        else:
+            srow = (torch.arange(pos + 1, pos + 1 + S) % 251).float()[None, None, :, None].expand(1, H, S, D).to(torch.bfloat16)
+            for layer in range(3):
+                a_cache.update_text(row, row, layer)
+                want_range = a_cache.attention_range(layer)
+                ks, _ = a_cache.get_summary_attention_kv(layer, srow, srow)
+                want_sum = ks[0, 0, :, 0].float().tolist()
+                a_cache.update_summary(srow, srow, layer)
+                # the same step from the rows `boundary_slots` names
+                assert b_cache.boundary_fits_one_piece(layer)
+                sl = b_cache.boundary_slots(layer, S)
+                for buf in (b_cache.key_cache[layer], b_cache.value_cache[layer]):
+                    _host_mover(row, buf, 1, 0, sl["text"])
+                    assert sl["attend"] == want_range
+                    if b_cache.is_large_window[layer]:
+                        _host_mover(srow, buf, S, 0, sl["spare"])
+                        got_sum = buf[0, 0, sl["spare"] - C:sl["spare"] + S, 0].float().tolist()
+                    else:
+                        _host_mover(srow, buf, S, 0, 0)
+                        got_sum = buf[0, 0, :S + C, 0].float().tolist()
+                        _host_mover(buf, buf, sl["flush_rows"], sl["flush_src"], sl["flush_dst"])
+                        _host_mover(srow, buf, S, 0, sl["append"])
+                    assert sorted(got_sum) == sorted(want_sum)
+            pos += 1 + S
+            n_boundaries += 1
+            a_cache.reset_chunk_counter()
+            b_cache.reset_chunk_counter()
+        n_text += 1
+        for name in counters:
+            va, vb = getattr(a_cache, name), getattr(b_cache, name)
+            if name == "_capacity":   # an append-only buffer also holds the step's spare rows
+                assert va[0] == vb[0] and all(x <= y for x, y in zip(va[1:], vb[1:]))
+            else:
+                assert va == vb, name
+        for layer in range(3):
+            a, e = a_cache.attention_range(layer)
+            assert b_cache.attention_range(layer) == (a, e)
+            assert torch.equal(a_cache.key_cache[layer][:, :, a:e], b_cache.key_cache[layer][:, :, a:e])
+            assert torch.equal(a_cache.value_cache[layer][:, :, a:e], b_cache.value_cache[layer][:, :, a:e])
+    assert n_boundaries >= 30
+
+
 def test_cache_summary_growth():
     """Summary region overflows its headroom -> buffer grows to the right, rows keep their place."""
     C, S = 2, 1

@@ -256,6 +256,7 @@ def test_gpu_module_config4_layer_shape():
     w = init_weights(cfg, "cuda", torch.bfloat16, 11)
     gpu = KsaQwen3ForCausalLM(cfg, w, HipOps())
     cpu = KsaQwen3ForCausalLM(cfg, convert_weights(w, "cpu", torch.float32), OracleOps())
+    gpu.BOUNDARY_GRAPH_AFTER = 0     # the graph run replays its boundary step too
     batch, n_prompt, n_new = 8, 300, 132
     ids = torch.randint(0, cfg.vocab_size, (batch, n_prompt), generator=torch.Generator().manual_seed(12))
     out_c, log_c = cpu.generate(ids, n_new, return_logits=True)
@@ -284,6 +285,7 @@ def test_gpu_graph_decode_equals_eager_decode():
                       summary_token_begin=1000)
     w = init_weights(cfg, "cuda", torch.bfloat16, 7)
     model = KsaQwen3ForCausalLM(cfg, w, HipOps())
+    model.BOUNDARY_GRAPH_AFTER = 0     # the boundary step is replayed from its own recording
     ids = torch.randint(0, cfg.vocab_size, (2, 200), generator=torch.Generator().manual_seed(9))
     n_new = 150
     out_e, log_e = model.generate(ids, n_new, return_logits=True)
@@ -315,3 +317,46 @@ def test_gpu_graph_decode_survives_buffer_growth():
     out_g, log_g = model.generate(ids, 60, forced=out_e[:, 140:], return_logits=True, use_graph=True)
     err = (log_e - log_g).abs().amax(dim=(0, 2))
     assert err.max().item() <= 1e-2 * log_e.abs().max().item(), err.tolist()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("S,indep,mix,after", [(1, False, 1.0, 0), (2, True, 0.35, 0), (2, False, 1.0, None)])
+def test_gpu_graph_boundary_steps_equal_eager(S, indep, mix, after):
+    """Chunk-boundary steps replayed from their own recording against the eager path: chunks of 8
+    tokens, 70 steps = 9 boundaries, a ring of two chunks (its write position wraps at every
+    second boundary) next to a ring of one and an unbounded layer, and head-rooms so small that
+    the summary region and the append-only buffers outgrow their buffers several times (each
+    growth moves the buffers, so both recordings are made again).  `after` = how many boundary
+    steps of a cache run eagerly before they are recorded (None: the class's own number, so the
+    switch happens in the middle of the run).  Tolerance as for the steps
+    inside a chunk: 1 % of the logit scale at every step (the two paths choose the decode
+    kernel's split count differently)."""
+    from ksa_amd.model import HipOps
+    cfg = tiny_config(summary_token_num=S, head_dim=128, summary_independent_parameters=indep, mix_coeff=mix,
+                      hidden_size=128, intermediate_size=256, summary_sliding_chunk_num=[2, 1, 1 << 20, 2])
+    w = init_weights(cfg, "cuda", torch.bfloat16, 5)
+    ops = HipOps()
+
+    class SmallHeadroom(ops.cache_cls):
+        _APPEND_HEADROOM = 6
+        _SUMMARY_INIT_CAP = 3
+    ops.cache_cls = SmallHeadroom
+    model = KsaQwen3ForCausalLM(cfg, w, ops)
+    if after is not None:
+        model.BOUNDARY_GRAPH_AFTER = after
+    replays = []
+    inner = model._replay
+    model._replay = lambda st, which, body, cache: (replays.append(which), inner(st, which, body, cache))[1]
+    ids = torch.randint(0, cfg.vocab_size, (2, 21), generator=torch.Generator().manual_seed(6))
+    n_new = 71
+    out_e, log_e = model.generate(ids, n_new, return_logits=True)
+    assert not replays
+    out_g, log_g = model.generate(ids, n_new, forced=out_e[:, 21:], return_logits=True, use_graph=True)
+    torch.cuda.synchronize()
+    n_b = sum(1 for t in range(21 + 1, 21 + n_new) if t % cfg.summary_chunk_size == 0)
+    assert n_b == 9 and replays.count("boundary") == n_b - model.BOUNDARY_GRAPH_AFTER, replays
+    assert replays.count("text") == n_new - 1 - n_b, replays
+    err = (log_e - log_g).abs().amax(dim=(0, 2))
+    scale = log_e.abs().max().item()
+    print(f"graph vs eager over {n_b} boundaries: max logit difference {err.max().item() / scale:.3e} of the logit scale")
+    assert err.max().item() <= 1e-2 * scale, (err / scale).tolist()
