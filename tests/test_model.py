@@ -360,3 +360,28 @@ def test_gpu_graph_boundary_steps_equal_eager(S, indep, mix, after):
     scale = log_e.abs().max().item()
     print(f"graph vs eager over {n_b} boundaries: max logit difference {err.max().item() / scale:.3e} of the logit scale")
     assert err.max().item() <= 1e-2 * scale, (err / scale).tolist()
+
+
+@pytest.mark.gpu
+def test_gpu_module_fp16():
+    """The module with fp16 weights and activations (every kernel of the step has an fp16 form):
+    the real attention shape, a 300-token prompt, 120 steps across a chunk boundary, launched
+    eagerly and replayed from the HIP graphs, against the fp32 host operators on the same
+    weights, teacher-forced.  Tolerance 0.3 % of the logit scale (measured 0.07-0.08 %; fp16
+    rounds eight times finer than bf16, whose bar is 1.5 %)."""
+    from ksa_amd.model import HipOps
+    from oracle.model_ops import OracleOps
+    cfg = tiny_config(summary_chunk_size=128, summary_token_num=8, head_dim=128, num_attention_heads=8,
+                      num_key_value_heads=2, hidden_size=256, intermediate_size=512, num_hidden_layers=3,
+                      summary_sliding_chunk_num=[1, 1 << 20, 1], vocab_size=1000, summary_token_begin=1000)
+    w = init_weights(cfg, "cuda", torch.float16, 21)
+    gpu = KsaQwen3ForCausalLM(cfg, w, HipOps())
+    gpu.BOUNDARY_GRAPH_AFTER = 0
+    cpu = KsaQwen3ForCausalLM(cfg, convert_weights(w, "cpu", torch.float32), OracleOps())
+    ids = torch.randint(0, cfg.vocab_size, (2, 300), generator=torch.Generator().manual_seed(22))
+    out_c, log_c = cpu.generate(ids, 120, return_logits=True)
+    for what, graph in (("eager", False), ("graph", True)):
+        _, log_g = gpu.generate(ids, 120, forced=out_c[:, 300:], return_logits=True, use_graph=graph)
+        assert log_g.dtype == torch.float32 and gpu.dtype == torch.float16
+        rel, agree, _ = _check_logits_and_tokens(log_g.cpu(), log_c, 3e-3, what)
+        print(f"fp16 {what}: max logit error {rel:.3e} of the logit scale, arg-max agreement {agree:.2f}")
