@@ -382,6 +382,19 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
     int seq_nxt = seq_chunk(64);
     uint32_t word_cur = kRegular ? tile_word(seq_cur) : 0u;
     uint32_t word_nxt = kRegular ? tile_word(seq_nxt) : 0u;
+    // Where a tile's first column stands in the period of C text + S summary columns of the
+    // in-line region, (n0 - P) mod (C + S) in [0, C + S): computed with the walk order, one
+    // division per lane and 64 tiles, so that the masked steps have none.
+    auto tile_phase = [&](int n) {
+        const int r = (n * kTileN - mk.P) % Bblk;
+        return r < 0 ? r + Bblk : r;
+    };
+    int phase_cur = tile_phase(seq_cur);
+    int phase_nxt = tile_phase(seq_nxt);
+    auto seq_phase = [&](int i, int it) {
+        const int src = (i >> 6) == (it >> 6) ? phase_cur : phase_nxt;
+        return __builtin_amdgcn_readlane(src, i & 63);
+    };
     // entry i in {it, .., it+3} while processing tile it
     auto seq = [&](int i, int it) {
         const int src = (i >> 6) == (it >> 6) ? seq_cur : seq_nxt;
@@ -468,24 +481,49 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
 
         if constexpr (kGeneral) {  // 64-bit visibility word per row
             const int kv = n0 + lane;
-            const int rel = kv - mk.P;
             const bool in = kv < mk.Sk;
             const uint64_t valid = __ballot(in);
-            const uint64_t text = __ballot(in && rel >= 0 && (rel % Bblk) < mk.C);
+            // text column: its offset in the period is below C.  phase + lane is below two periods
+            // when a period holds a tile's 64 columns (any real chunk size).
+            int o = seq_phase(it, it) + lane;
+            if (Bblk >= kTileN) o -= o >= Bblk ? Bblk : 0;
+            else o %= Bblk;
+            const uint64_t text = __ballot((int)in & (int)(kv >= mk.P) & (int)(o < mk.C));
             const uint64_t fa = prefix_mode ? valid : (valid & ~text);
+            // bits [lo, hi) of a 64-bit word, without a branch
+            auto range_bits = [](int lo, int hi) {
+                lo = max(lo, 0);
+                hi = max(hi, 0);
+                const uint64_t below_hi = hi >= 64 ? ~0ull : ~(~0ull << hi);
+                const uint64_t from_lo = lo >= 64 ? 0ull : (~0ull << lo);
+                return below_hi & from_lo;
+            };
+            // -inf where the word has a 0: one bit-field extract (0 or all ones) and one bit-field
+            // insert per element, no compare; a half whose 16 bits are set in every lane that sees
+            // anything of the tile is left alone (the 8 summary columns that a tile below the
+            // diagonal hides from text rows lie in one half).
+            auto mask_half = [](floatx16& sc, uint32_t w, bool any) {
+                if (__ballot(any && (w & 0x0f0f0f0fu) != 0x0f0f0f0fu) == 0ull) return;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const uint32_t m = (uint32_t)__builtin_amdgcn_sbfe((int)w, 8 * (i / 4) + (i % 4), 1);
+                    sc[i] = __uint_as_float((__float_as_uint(sc[i]) & m) | (0xff800000u & ~m));
+                }
+            };
+            // (uniform) a tile of the in-line region behind a prefix: no row's [0, xa) reaches it
+            const bool no_xa = prefix_mode && n0 >= mk.P;
 #pragma unroll
             for (int r = 0; r < RB; ++r) {
                 const uint64_t fb = rv[r].b_text ? text : valid;
-                const uint64_t bits = (ksa_range_bits(-n0, rv[r].xa - n0) & fa) |
-                                      (ksa_range_bits(rv[r].blo - n0, rv[r].bhi - n0) & fb);
+                uint64_t bits = range_bits(rv[r].blo - n0, rv[r].bhi - n0) & fb;
+                if (!no_xa) bits |= range_bits(-n0, rv[r].xa - n0) & fa;
+                // a row that sees nothing of the tile loses it through its reference (infinite:
+                // every probability 0) and does not keep a half from being skipped
+                const bool any = bits != 0ull;
+                row_vis[r] = any;
                 const uint64_t sh = bits >> (4 * lh);
-                const uint32_t w0 = (uint32_t)sh, w1 = (uint32_t)(sh >> 32);
-#pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const uint32_t bit = 1u << (8 * (i / 4) + (i % 4));
-                    scur[r][0][i] = (w0 & bit) ? scur[r][0][i] : -INFINITY;
-                    scur[r][1][i] = (w1 & bit) ? scur[r][1][i] : -INFINITY;
-                }
+                mask_half(scur[r][0], (uint32_t)sh, any);
+                mask_half(scur[r][1], (uint32_t)(sh >> 32), any);
             }
         }
 
@@ -618,8 +656,10 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
         if ((it & 63) == 63) {  // roll the index chunk
             seq_cur = seq_nxt;
             word_cur = word_nxt;
+            phase_cur = phase_nxt;
             seq_nxt = seq_chunk(it + 1 + 64);
             word_nxt = kRegular ? tile_word(seq_nxt) : 0u;
+            phase_nxt = tile_phase(seq_nxt);
         }
     };
 
@@ -649,6 +689,8 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
         seq_nxt = seq_chunk(64);
         word_cur = kRegular ? tile_word(seq_cur) : 0u;
         word_nxt = kRegular ? tile_word(seq_nxt) : 0u;
+        phase_cur = tile_phase(seq_cur);
+        phase_nxt = tile_phase(seq_nxt);
 #pragma unroll
         for (int r = 0; r < RB; ++r) {
             m_ref[r] = -1e30f;  // finite: the first rescale multiplies the zero accumulators by 0
