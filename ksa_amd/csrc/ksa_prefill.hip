@@ -488,7 +488,7 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
             int o = seq_phase(it, it) + lane;
             if (Bblk >= kTileN) o -= o >= Bblk ? Bblk : 0;
             else o %= Bblk;
-            const uint64_t text = __ballot((int)in & (int)(kv >= mk.P) & (int)(o < mk.C));
+            const uint64_t text = valid & __ballot(kv >= mk.P) & __ballot(o < mk.C);
             const uint64_t fa = prefix_mode ? valid : (valid & ~text);
             // bits [lo, hi) of a 64-bit word, without a branch
             auto range_bits = [](int lo, int hi) {
@@ -501,7 +501,8 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
             // -inf where the word has a 0: one bit-field extract (0 or all ones) and one bit-field
             // insert per element, no compare; a half whose 16 bits are set in every lane that sees
             // anything of the tile is left alone (the 8 summary columns that a tile below the
-            // diagonal hides from text rows lie in one half).
+            // diagonal hides from text rows lie in one half; skipping by groups of 8 keys inside a
+            // half as well measured slower: cfg 2 -0.3 %, cfg 1 -1.1 %).
             auto mask_half = [](floatx16& sc, uint32_t w, bool any) {
                 if (__ballot(any && (w & 0x0f0f0f0fu) != 0x0f0f0f0fu) == 0ull) return;
 #pragma unroll
