@@ -438,10 +438,20 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
         if constexpr (RB != 1) ksa_mfma_settle();
     };
 
+    // MFMA operands that come from LDS travel through a rolling queue of kQueue fragments that
+    // runs across the steps: see `step`.
+    constexpr int kQueue = 4;
+#ifndef KSA_PREFILL_BEHIND
+#define KSA_PREFILL_BEHIND 4
+#endif
+    constexpr int kBehind = KSA_PREFILL_BEHIND;  // MFMAs of the second product behind the step's barrier
+    static_assert(kBehind >= 1 && kBehind <= kQueue, "fragments behind the barrier come from the queue");
+    u32x4 fq[kQueue];
     // One pipeline step for tile `it` (parity tag = it % 2): its scores are in `scur`; the
-    // scores of tile it+1 are produced into `snext`.  On entry the fills of K(it+1) and V(it)
-    // have landed; the barrier publishes them and frees the other two buffers, which this step
-    // refills with K(it+2) and V(it+1) while it computes.
+    // scores of tile it+1 are produced into `snext`.  On entry K(it+1) and V(it) are in LDS and
+    // published (the previous step's barrier, or the prologue's), the first operands of the score
+    // product are in the queue, and the other two buffers are free: this step refills them with
+    // K(it+2) and V(it+1) while it computes and publishes them with its own barrier near its end.
     // `quick`: a row is visible as a whole iff it is a text row (leading prefix tiles).
     auto step = [&](auto safe_tag, auto general_tag, auto parity_tag, int it, floatx16 (&scur)[RB][2],
                     floatx16 (&snext)[RB][2], bool quick) __attribute__((always_inline)) {
@@ -451,21 +461,23 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
         const int n0 = seq(it, it) * kTileN;
         // Past the end of the walk the pipeline keeps running on the last tile (fills) and
         // on stale LDS contents (scores); those results are never used.
-        // fills: K(it+2) in the score stage, V(it+1) in the second-product stage
+        // fills: K(it+2) and V(it+1), both issued in the first slots of the score stage
         const int ik = min(it + 2, ntiles - 1), iv = min(it + 1, ntiles - 1);
         const int nk = seq(ik, it), nv = seq(iv, it);
         const uint32_t wk = seq_word(ik, it), wv = seq_word(iv, it);
         bool row_vis[RB];
 #pragma unroll
         for (int r = 0; r < RB; ++r) row_vis[r] = quick ? rv[r].b_text : true;
-        wg_barrier();
 
         // MFMA operands that come from LDS travel through a rolling queue of kQueue fragments:
         // the read for operand j + kQueue is issued right behind the MFMAs of operand j, through
-        // the score product (K fragments), across its end (the first V fragments) and through
-        // the second product, so every read has kQueue operands' worth of MFMAs plus the vector
-        // work between them to land.
-        constexpr int kQueue = 4;
+        // the score product (K fragments), across its end (the first V fragments), through the
+        // second product and across the end of the step (the first K fragments of the next step),
+        // so every read has kQueue operands' worth of MFMAs plus the vector work between them to
+        // land.  The step's barrier stands in front of the last kQueue MFMAs of the second
+        // product: by then every fragment this step takes from LDS is in registers, the barrier
+        // publishes the tiles filled during the step, and the MFMAs behind it cover the reads
+        // of the next step's first fragments.
         constexpr int NQK = 2 * KS;   // K fragments: contraction step s = j / 2, key block kb = j % 2
         constexpr int NPV = 4 * DB;   // V fragments: key step ks = j / DB, dim block j % DB
         const uint16_t* ksrc = PAR ? Ks0 : Ks1;   // K(it+1)
@@ -474,9 +486,6 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
         uint16_t* vdst = PAR ? Vs0 : Vs1;         // <- V(it+1)
         auto kfrag = [&](int j) { return read_k(ksrc, j); };
         auto vfrag = [&](int j) { return read_v(vsrc, j); };
-        u32x4 fq[kQueue];
-#pragma unroll
-        for (int j = 0; j < kQueue; ++j) fq[j] = kfrag(j);
         __builtin_amdgcn_sched_barrier(0);
 
         if constexpr (kGeneral) {  // 64-bit visibility word per row
@@ -609,7 +618,7 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
         constexpr int CPM = 16 / NQK;            // probability pairs per score MFMA
         constexpr int kLead = 3;
         constexpr int NM = NQK * RB;
-        static_assert(KLD <= NM && KLD <= NPV, "one fill per MFMA slot at most");
+        static_assert(2 * KLD <= NM, "one fill per MFMA slot at most");
 #pragma unroll
         for (int vt = 0; vt < kLead; ++vt) prob_slot(vt);
         __builtin_amdgcn_sched_barrier(0);
@@ -630,6 +639,7 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
 #pragma unroll
                 for (int vt = kLead + m * CPM; vt < kLead + (m + 1) * CPM; ++vt) prob_slot(vt);
                 if (m < KLD) fill1(kbase, kdst, kcol, nk, wk, m);
+                else if (m < 2 * KLD) fill1(vbase, vdst, vcol, nv, wv, m - KLD);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -644,16 +654,22 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
         // O^T += V^T P^T
 #pragma unroll
         for (int j = 0; j < NPV; ++j) {
+            if (j == NPV - kBehind) {
+                fills_done();
+                wg_barrier();
+                // the next step's fragments whose queue places came free in front of the barrier
+#pragma unroll
+                for (int t = NPV; t < NPV - kBehind + kQueue; ++t) fq[t % kQueue] = read_k(kdst, t - NPV);
+            }
 #pragma unroll
             for (int r = 0; r < RB; ++r) {
                 if constexpr (RB == 1) oacc[r][j % DB] = Ops::mfma(fq[j % kQueue], pf[r][j / DB], oacc[r][j % DB]);
                 else Ops::mfma_a(oacc[r][j % DB], fq[j % kQueue], pf[r][j / DB]);
             }
             if (j + kQueue < NPV) fq[j % kQueue] = vfrag(j + kQueue);
-            if (j < KLD) fill1(vbase, vdst, vcol, nv, wv, j);
+            else if (j >= NPV - kBehind) fq[j % kQueue] = read_k(kdst, j + kQueue - NPV);
             __builtin_amdgcn_sched_barrier(0);
         }
-        fills_done();
         if ((it & 63) == 63) {  // roll the index chunk
             seq_cur = seq_nxt;
             word_cur = word_nxt;
@@ -709,6 +725,8 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
             fills_done();
             __syncthreads();
             scores(s0, Ks0);
+#pragma unroll
+            for (int j = 0; j < kQueue; ++j) fq[j] = read_k(Ks1, j);  // the first step's first operands
             if constexpr (!kSafe) {
 #pragma unroll
                 for (int r = 0; r < RB; ++r) {
