@@ -22,7 +22,9 @@
 // soft-max of tile i, one MFMA and one pair of probabilities per time slot, so that matrix
 // and vector work of one wave overlap; K therefore runs one tile ahead of V through LDS.
 // All MFMA operands that come from LDS pass through a small rolling queue of fragments that
-// is refilled right behind each MFMA.
+// is refilled right behind each MFMA and runs across the steps; the one workgroup barrier of a
+// step stands in front of the last MFMAs of its second product, which then cover the reads of
+// the next step's first fragments.
 //
 // Masking.  The walk has two phases that are uniform for the workgroup.  Phase A holds
 // the tiles that need no per-element mask: the leading partial tiles below every text
