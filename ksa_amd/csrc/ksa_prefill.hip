@@ -729,6 +729,8 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
             scores(s0, Ks0);
 #pragma unroll
             for (int j = 0; j < kQueue; ++j) fq[j] = read_k(Ks1, j);  // the first step's first operands
+            // the first step refills K(0)'s buffer at once: every wave must be done reading it
+            wg_barrier();
             if constexpr (!kSafe) {
 #pragma unroll
                 for (int r = 0; r < RB; ++r) {
