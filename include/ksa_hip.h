@@ -263,11 +263,21 @@ int ksa_gemm_rows_gate_up_silu(const void* x, const void* w, void* out, int M, i
  *   workspace: ksa_mlp_rows_workspace_bytes(H, I) bytes, 16-byte aligned, ZEROED ONCE by the caller
  *   before its first use and then left alone (its counting words go up from launch to launch);
  *   it belongs to one device and one pair (H, I), and launches that share it must not overlap.
- *   Every wait inside the kernel is bounded: a workgroup that does not see its tiles arrive within
- *   about a second gives up, the output of that launch is unusable and the 8-byte word at
- *   ksa_mlp_rows_status_offset() of the workspace reads 1 - the caller then zeroes the workspace
- *   again.  KSA_ERR_UNSUPPORTED for sizes outside the above: use
- *   the two separate calls. */
+ *   M may differ from launch to launch on one workspace, and launches with and without the norm
+ *   stage of ksa_add_rmsnorm_mlp_rows may be mixed on it.
+ *   What the kernel relies on: the workgroups of a launch are STARTED IN THE ORDER OF THEIR NUMBERS
+ *   (a waiting workgroup depends only on workgroups with lower numbers, so those have been started
+ *   and can finish).  HIP does not promise that order; the hardware dispatcher of gfx950 keeps it
+ *   for a one-dimensional grid.  It can also be defeated from outside: a second launch on the same
+ *   workspace that runs at the same time (another stream), or a CU mask / a co-tenant that leaves
+ *   so few CUs that the launch takes longer than the bound below.  Every wait inside the kernel is
+ *   therefore bounded: a workgroup that does not see its tiles arrive within
+ *   about a second gives up, every workgroup that waits after it leaves at once, the launch ends
+ *   normally, its output is unusable and the 8-byte word at
+ *   ksa_mlp_rows_status_offset() of the workspace reads 1.  The caller then waits for the device to
+ *   be idle, zeroes the workspace again and repeats the work with the two separate calls
+ *   (ksa_gemm_rows_gate_up_silu + ksa_gemm_rows), which depend on no such order.
+ *   KSA_ERR_UNSUPPORTED for sizes outside the above: use the two separate calls. */
 int ksa_mlp_rows_down_splits(int H, int I);
 size_t ksa_mlp_rows_workspace_bytes(int H, int I);
 size_t ksa_mlp_rows_status_offset(void);

@@ -45,11 +45,13 @@ namespace {
 constexpr int kSlices = 4;        // K slices of the hidden size = waves per gate / up half
 constexpr int kTileCols = 16;     // columns of the activation per gate | up workgroup (8: same time, twice the reads of x)
 constexpr int kWordStride = 64;   // 64-bit words are 512 bytes apart
-// words: [0] launches so far, [1] down workgroups done, [2] status, [4 .. 11] rows of the norm stage done
-// (eight copies, a gate | up workgroup watches copy number % 8: hundreds of workgroups polling one
-// word would queue at it), [12 + c] tiles of chunk c stored
-constexpr int kWordLaunches = 0, kWordDone = 1, kWordStatus = 2, kWordHeadLaunches = 3, kWordHead0 = 4, kHeadCopies = 8,
-              kWordChunk0 = 12;  // ([3] launches with a norm stage: those without one do not move the words [4 .. 11])
+// words: [0] launches so far, [1] down workgroups done, [2] status, [3] rows of the norm stages of all past
+// launches (a launch may have any number of rows, and one without a norm stage has none: the target of a
+// wait is this word plus the rows of the launch itself), [4 .. 11] rows of the norm stage done (eight copies,
+// a gate | up workgroup watches copy number % 8: hundreds of workgroups polling one word would queue at it),
+// [12 + c] tiles of chunk c stored (the same number in every launch: it depends on I alone)
+constexpr int kWordLaunches = 0, kWordDone = 1, kWordStatus = 2, kWordHeadRows = 3, kWordHead0 = 4, kHeadCopies = 8,
+              kWordChunk0 = 12;
 constexpr int kMaxChunks = 52;    // K of the down projection up to 26624
 constexpr int kSyncWords = kWordStride * (kWordChunk0 + kMaxChunks);
 
@@ -165,11 +167,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
             st_agent(hp, (unsigned long long)o[0] | ((unsigned long long)o[1] << 32));
             st_agent(hp + 1, (unsigned long long)o[2] | ((unsigned long long)o[3] << 32));
         }
-        __syncthreads();  // every store of the workgroup is issued and counted off (s_waitcnt before the barrier)
-        if (tid < kHeadCopies) {
-            __builtin_amdgcn_s_waitcnt(0);
-            add_agent(p.sync + kWordStride * (kWordHead0 + tid), 1ull);
-        }
+        // Every thread waits until its own stores have left (they write through to memory), and only then
+        // joins the barrier: the barrier itself does not wait for the stores of the other waves.
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+        if (tid < kHeadCopies) add_agent(p.sync + kWordStride * (kWordHead0 + tid), 1ull);
         return;
     }
     const int bid = blockIdx.x - p.head;  // number among the workgroups of the two products
@@ -194,10 +196,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
         if (p.head > 0) {
             // the rows of the norm stage: wait for its count, then fetch them past this XCD's L2
             if (tid == 0) {
-                const unsigned long long launch = ld_agent(p.sync + kWordStride * kWordHeadLaunches);
+                const unsigned long long before = ld_agent(p.sync + kWordStride * kWordHeadRows);
                 unsigned long long* word = p.sync + kWordStride * (kWordHead0 + (bid % kHeadCopies));
                 unsigned long long* status = p.sync + kWordStride * kWordStatus;
-                const unsigned long long want = (launch + 1) * (unsigned long long)p.head;
+                const unsigned long long want = before + (unsigned long long)p.head;
                 unsigned spins = 0;
                 int fail = 0;
                 while (ld_agent(word) < want) {
@@ -351,7 +353,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
         const unsigned long long nd = (unsigned long long)p.GR * p.KC;
         if (add_agent(p.sync + kWordStride * kWordDone, 1ull) == (launch + 1) * nd - 1) {
             add_agent(p.sync + kWordStride * kWordLaunches, 1ull);
-            if (p.head > 0) add_agent(p.sync + kWordStride * kWordHeadLaunches, 1ull);
+            if (p.head > 0) add_agent(p.sync + kWordStride * kWordHeadRows, (unsigned long long)p.head);
         }
     }
 }

@@ -81,9 +81,15 @@ def gate_up_silu_rows(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     return out.view(*x.shape[:-1], I)
 
 
+class MlpRowsTimeout(RuntimeError):
+    """A `ksa_mlp_rows` / `ksa_add_rmsnorm_mlp_rows` launch gave up waiting inside the kernel: what was
+    computed since the last clean check is not valid."""
+
+
 class MlpRowsWorkspace:
     """Barrier words and the activation buffer of `mlp_rows` for one (device, hidden size, MLP size):
-    zeroed once, then shared by every layer's call on that stream (the calls run one after the other)."""
+    zeroed once, then shared by every layer's call on that stream (the calls run one after the other,
+    with any number of rows each)."""
 
     def __init__(self, H: int, I: int, device):
         L = _lib.lib()
@@ -92,11 +98,15 @@ class MlpRowsWorkspace:
         self._status = self.buf[L.ksa_mlp_rows_status_offset():][:8].view(torch.int64)
 
     def failed(self) -> bool:
-        """True if a launch gave up waiting at a grid barrier (synchronises; the workspace is zeroed
-        again so that it can be used further)."""
+        """True if a launch gave up waiting inside the kernel.  Waits for the whole device to be idle
+        first (no launch on the workspace may be in flight, on any stream, when its words are read or
+        cleared); after a failure the workspace is zeroed again so that it can be used further.
+        Recorded graphs that launch on it stay valid (the buffer does not move)."""
+        torch.cuda.synchronize(self.buf.device)
         bad = bool(self._status.item() != 0)
         if bad:
             self.buf.zero_()
+            torch.cuda.synchronize(self.buf.device)
         return bad
 
 

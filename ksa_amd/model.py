@@ -145,7 +145,10 @@ class HipOps:
         self._argmax_rows = elementwise.argmax_rows
         self._max_rows = gemm.MAX_ROWS
         self._gemm = gemm
+        self.timeout_error = gemm.MlpRowsTimeout
         self._mlp_ws = {}   # (device, H, I) -> MlpRowsWorkspace, see `mlp_rows`
+        # False: the MLP of a decode step runs as separate launches (set after a one-launch MLP timed out)
+        self.mlp_one_launch = True
 
     def decode(self, q, kbuf, vbuf, start, end, scale):
         return self._decode(q, kbuf, vbuf, start, end, scale=scale)
@@ -170,7 +173,7 @@ class HipOps:
         partial sums of the down projection; None when the shape is outside what that kernel takes."""
         rows = x.numel() // x.shape[-1]
         H, I = x.shape[-1], w_down.shape[1]
-        if not self._gemm.mlp_rows_supported(rows, H, I):
+        if not self.mlp_one_launch or not self._gemm.mlp_rows_supported(rows, H, I):
             return None
         return self._gemm.mlp_rows(x, w_gate_up, w_down, self.prepare_mlp_rows(H, I, x.device))
 
@@ -178,7 +181,7 @@ class HipOps:
         """(residual + o_proj output, down(SiLU(gate(h)) * up(h)) for h = norm of that sum) in one launch,
         from the K-split partial sums of the o projection; None when the shapes are outside what the
         kernel takes."""
-        if not isinstance(o_partials, self._gemm.SplitKPartials):
+        if not self.mlp_one_launch or not isinstance(o_partials, self._gemm.SplitKPartials):
             return None
         H, I = residual.shape[-1], w_down.shape[1]
         if not self._gemm.mlp_rows_supported(o_partials.rows, H, I) or H > 4096:
@@ -187,8 +190,19 @@ class HipOps:
                                                self.prepare_mlp_rows(H, I, residual.device))
 
     def mlp_rows_failed(self):
-        """True if a `mlp_rows` launch gave up waiting (synchronises); see `MlpRowsWorkspace.failed`."""
-        return any(ws.failed() for ws in self._mlp_ws.values())
+        """True if a `mlp_rows` launch gave up waiting since the last call (waits for the device; every
+        workspace is looked at and, where needed, cleared: see `MlpRowsWorkspace.failed`)."""
+        return any([ws.failed() for ws in self._mlp_ws.values()])
+
+    def check_mlp_rows(self):
+        """Raises `MlpRowsTimeout` if a one-launch MLP gave up waiting since the last check, and from
+        then on runs the MLP of a decode step as separate launches, which depend on nothing but the
+        order of launches on a stream."""
+        if self.mlp_one_launch and self.mlp_rows_failed():
+            self.mlp_one_launch = False
+            raise self._gemm.MlpRowsTimeout(
+                "ksa_mlp_rows: a workgroup gave up waiting for the tiles it depends on; the steps since the "
+                "last check are not valid.  The one-launch MLP is switched off for this operator set.")
 
     def gate_up_act(self, x, weight):
         """SiLU(x W_gate^T) * (x W_up^T) for the fused gate | up matrix: one kernel for the few rows of
@@ -403,6 +417,24 @@ class KsaQwen3ForCausalLM:
         return self._logits(x[:, last_text:last_text + 1], delta[:, last_text:last_text + 1]), cache
 
     # ---- decode ----------------------------------------------------------------------
+    def check_steps(self, cache=None):
+        """Raises (`ops.timeout_error`) if a launch of the decode steps since the last check reported
+        that it could not finish its work (the one-launch MLP's bounded waits); the operator set then
+        uses the separate launches from there on, and the recordings of `cache` that hold the
+        one-launch form are dropped.  Waits for the device.  `decode_step` and `decode_step_graph`
+        call this at every chunk boundary, `generate` also at its end, and repeats the call."""
+        chk = getattr(self.ops, "check_mlp_rows", None)
+        if chk is None:
+            return
+        try:
+            chk()
+        except getattr(self.ops, "timeout_error", ()):
+            st = getattr(cache, "_ksa_graph_state", None)
+            if st is not None:
+                st["graphs"].clear()
+            self._graph_warm = set()   # the other path's launches get their eager run before a recording
+            raise
+
     @torch.no_grad()
     def decode_step(self, token_ids: torch.Tensor, cache):
         """token_ids [b, 1] (the newest text token) -> logits [b, 1, vocab].  When the token
@@ -413,6 +445,8 @@ class KsaQwen3ForCausalLM:
         b = token_ids.shape[0]
         true_tokens = cache.get_true_token_num()
         boundary = cache.get_cur_chunk_size() == C - 1
+        if boundary:
+            self.check_steps(cache)   # before the step that cannot be undone (it flushes the chunk)
         ids = token_ids.to(self.device)
         if boundary:
             sids = torch.arange(S, device=self.device, dtype=ids.dtype) + cfg.summary_token_begin
@@ -624,6 +658,7 @@ class KsaQwen3ForCausalLM:
             cache._ksa_graph_state = st
         kinds = [1 if cache.is_large_window[li] else 0 for li in range(nl)]
         if cache.get_cur_chunk_size() == C - 1:
+            self.check_steps(cache)
             # recorded: a boundary step whose flush is one whole chunk in one piece (every boundary of
             # a cache filled by `prefill`), once the cache has seen enough of them; else eagerly
             st["boundaries"] = st.get("boundaries", 0) + 1
@@ -705,7 +740,15 @@ class KsaQwen3ForCausalLM:
         """Greedy decoding.  Returns ids [b, n + max_new_tokens] (and the logits of every step,
         [b, max_new_tokens, vocab], on request).  `forced` [b, max_new_tokens] replaces the
         arg-max token fed back at every step (teacher forcing, for comparing two runs).
-        `use_graph` replays the decode steps from HIP graphs (`decode_step_graph`)."""
+        `use_graph` replays the decode steps from HIP graphs (`decode_step_graph`).
+        If a launch reports that it could not finish (`check_steps`), the whole call is repeated
+        once on the separate-launch path, which `check_steps` has switched to."""
+        try:
+            return self._generate(input_ids, max_new_tokens, forced, return_logits, use_graph)
+        except getattr(self.ops, "timeout_error", ()):
+            return self._generate(input_ids, max_new_tokens, forced, return_logits, use_graph)
+
+    def _generate(self, input_ids, max_new_tokens, forced, return_logits, use_graph):
         logits, cache = self.prefill(input_ids)
         out, steps = [], []
         for t in range(max_new_tokens):
@@ -718,7 +761,5 @@ class KsaQwen3ForCausalLM:
                 feed = nxt if forced is None else forced[:, t:t + 1].to(self.device)
                 logits = self.decode_step_graph(feed, cache) if use_graph else self.decode_step(feed, cache)
         ids = torch.cat([input_ids.to(self.device)] + out, dim=1)
-        if hasattr(self.ops, "mlp_rows_failed") and self.ops.mlp_rows_failed():
-            raise RuntimeError("ksa_mlp_rows: a workgroup gave up waiting for the activation tiles of its chunk; "
-                               "the tokens of this call are not valid")
+        self.check_steps(cache)
         return (ids, torch.stack(steps, dim=1)) if return_logits else ids

@@ -78,3 +78,104 @@ def test_decode_equals_prefill_row(C, S, scn, n_prefill):
                 cache.update_summary(rows(K, pos, pos + S), rows(V, pos, pos + S), layer)
             pos += S
             cache.reset_chunk_counter()
+
+
+def test_cache_handoff_at_1024_chunks():
+    """The hand-off prefill -> `reorganize_after_prefill` -> decode at the decode benchmark's own size:
+    1024 complete chunks (C = 128, S = 8, a ring of 4 chunks, 32 / 8 heads, batch 2 with different rows
+    per sequence), a small-window layer next to a large-window one (whose reorganisation gathers the
+    131072 text rows out of 139264).  Then C + 3 decode steps across one chunk boundary through
+    `update_text`, `get_summary_attention_kv` and `update_summary`.  Every step's output (decode kernel
+    over `attention_range` of the whole buffer) is compared with
+      (a) the masked-attention oracle's row for that position on the full in-line sequence, and
+      (b) the prefill kernel's own row for that position (one prefill launch over the final sequence),
+    which is the decode == prefill-row invariant at this size.  The buffer capacity and the attended
+    range are the reference's closed forms (modeling_qwen3sa.py:265-266, :421-431): capacity
+    S + C + 4 C + 8192 + max(512, 8192 + 256) = 17288, range (136 - rows of the chunk, 8808) until the
+    boundary, (…, 8816) after it."""
+    import ksa_amd
+    dev = torch.device("cuda")
+    C, S, scn, Hq, Hkv, D, bsz = 128, 8, 4, 32, 8, 128, 2
+    B = C + S
+    n_chunks = 1024
+    n_prefill = n_chunks * C
+    steps = C + 3
+    Sq = n_chunks * B
+    Stot = Sq + B + 3                      # prefill + one more chunk with its summaries + 3 text rows
+    g = torch.Generator().manual_seed(2)
+    K = torch.randn(bsz, Stot, Hkv, D, generator=g).bfloat16()
+    V = torch.randn(bsz, Stot, Hkv, D, generator=g).bfloat16()
+    Q = torch.randn(bsz, Stot, Hq, D, generator=g).bfloat16()
+    Kd, Vd, Qd = K.to(dev), V.to(dev), Q.to(dev)
+
+    cfg = types.SimpleNamespace(summary_chunk_size=C, summary_token_num=S, num_hidden_layers=2)
+    cache = ksa_amd.Qwen3RingBufferCache(cfg, [scn, 10 ** 6])
+    sp = torch.from_numpy(O.summary_positions(Sq, C, S))[None].to(dev)
+
+    def rows(t, a, b):       # [bsz, heads, n, D] view as the HF model hands them in
+        return t[:, a:b].permute(0, 2, 1, 3)
+
+    for layer in range(2):
+        cache.update(rows(Kd, 0, Sq), rows(Vd, 0, Sq), layer, {"summary_mask": sp})
+    cache.reorganize_after_prefill(sp)
+    assert cache._capacity[0] == 17288 and cache.key_cache[0].shape == (bsz, Hkv, 17288, D)
+    assert cache._text_len[1] == n_prefill and cache.attention_range(1) == (0, n_prefill)
+    assert cache.attention_range(0) == (136, 8808)
+    # the gather itself, bit for bit: ring rows = text of the last four chunks, summaries in order
+    ring = cache.key_cache[0][:, :, S + C:S + C + scn * C]
+    want_ring = torch.cat([rows(Kd, c * B, c * B + C) for c in range(n_chunks - scn, n_chunks)], dim=2)
+    assert torch.equal(ring, want_ring)
+    sums = cache.value_cache[0][:, :, S + C + scn * C:S + C + scn * C + n_chunks * S]
+    assert torch.equal(sums, rows(Vd, 0, Sq)[:, :, sp[0]])
+    assert torch.equal(cache.key_cache[1][:, :, :n_prefill], rows(Kd, 0, Sq)[:, :, ~sp[0]])
+
+    class M:
+        num_key_value_groups = Hq // Hkv
+
+    pos, n_text = Sq, n_prefill
+    got = [[], []]
+    positions = []
+    for step in range(steps):
+        for layer in range(2):
+            cache.update_text(rows(Kd, pos, pos + 1), rows(Vd, pos, pos + 1), layer)
+            a, e = cache.attention_range(layer)
+            if layer == 0:
+                cbl = cache._chunk_buf_len[0]
+                assert (a, e) == (136 - cbl, 8808 if step < C else 8816), (step, a, e)
+            o = ksa_amd.ksa_decode(rows(Qd, pos, pos + 1), cache.key_cache[layer], cache.value_cache[layer], a, e)
+            if step in (0, C - 1, C):   # the reference's own call form: a slice of the cache
+                kf, vf = cache.get_attention_kv(layer)
+                o2, _ = ksa_amd.decode_attention_forward(M(), rows(Qd, pos, pos + 1), kf, vf, None, scaling=D ** -0.5)
+                assert (o2.float() - o.float()).abs().max().item() <= 1e-2
+            got[layer].append(o[:, 0])
+        positions.append(pos)
+        n_text += 1
+        pos += 1
+        if n_text % C == 0:
+            for layer in range(2):
+                ks, vs = cache.get_summary_attention_kv(layer, rows(Kd, pos, pos + S), rows(Vd, pos, pos + S))
+                so, _ = ksa_amd.decode_attention_forward(M(), rows(Qd, pos, pos + S), ks, vs, None, scaling=D ** -0.5)
+                sel = np.r_[pos:pos + S, pos - C:pos]
+                wq = c_oracle.decode(to_np(Q[:, pos:pos + S]).transpose(0, 2, 1, 3),
+                                     to_np(K[:, sel]).transpose(0, 2, 1, 3), to_np(V[:, sel]).transpose(0, 2, 1, 3),
+                                     0, len(sel))
+                assert np.abs(to_np(so) - wq).max() <= 2e-2
+                cache.update_summary(rows(Kd, pos, pos + S), rows(Vd, pos, pos + S), layer)
+            pos += S
+            cache.reset_chunk_counter()
+    assert cache._n_summaries[0] == (n_chunks + 1) * S and cache._window_write_ptr[0] == C % (scn * C)
+    n_used = pos
+    prow = np.array(positions, np.int32)
+    spf = torch.from_numpy(O.summary_positions(n_used, C, S)).to(dev)
+    for layer, window in ((0, scn), (1, 10 ** 6)):
+        dec = torch.stack(got[layer], dim=1)                     # [bsz, steps, Hq, D]
+        for b in range(bsz):
+            want, _ = c_oracle.attention_rows(to_np(Q[b, :n_used]), to_np(K[b, :n_used]), to_np(V[b, :n_used]),
+                                              C, S, window, rows=prow)
+            err = np.abs(to_np(dec[b]) - want).max()
+            assert err <= 2e-2, (layer, b, err)
+            pre, _ = ksa_amd.summary_attn_func(Qd[b:b + 1, :n_used], Kd[b:b + 1, :n_used], Vd[b:b + 1, :n_used],
+                                               C, S, window, summary_pos=spf)
+            perr = (pre[0, torch.as_tensor(prow, device=dev).long()].float() - dec[b].float()).abs().max().item()
+            print(f"layer {layer} seq {b}: decode vs oracle {err:.2e}, decode vs prefill kernel row {perr:.2e}")
+            assert perr <= 2e-2, (layer, b, perr)

@@ -203,3 +203,82 @@ def test_gpu_add_rmsnorm_mlp_rows_one_launch(dtype, M, H, I):
         assert (sum_new - sum_ref).abs().max().item() <= 4e-3 * sum_ref.abs().max().item() + 1e-5
         if rep == 1:
             mlp_rows(h_ref, w_gu, w_dn, ws)
+
+
+def _o_partials(M, H, dtype, dev, g):
+    """The K-split partial sums of an o projection for M rows, as `linear_rows(..., defer=True)` leaves them."""
+    from ksa_amd.gemm import SplitKPartials, linear_rows
+    attn = torch.randn(1, M, 4096, generator=g).to(dtype).to(dev)
+    w_o = (torch.randn(H, 4096, generator=g) * 0.03).to(dtype).to(dev)
+    o = linear_rows(attn, w_o, defer=True)
+    assert isinstance(o, SplitKPartials)
+    return o
+
+
+@pytest.mark.gpu
+def test_gpu_mlp_rows_row_count_changes_on_one_workspace():
+    """Launches with 8, then 2, then 8, then 1, then 16 rows on ONE workspace, with and without the norm
+    stage: the words that the waits compare against must not depend on the row counts of earlier
+    launches.  (With a target of "launches x rows of this launch" a 2-row launch behind 8-row ones would
+    not wait for its norm stage at all and read the rows of an earlier launch.)  Every result is compared
+    with the same call on a fresh workspace, bit for bit, and the norm stage's input differs from launch
+    to launch so that stale rows cannot pass."""
+    from ksa_amd.gemm import MlpRowsWorkspace, add_rmsnorm_mlp_rows, mlp_rows
+    dtype, dev = torch.bfloat16, torch.device("cuda")
+    H, I = 2560, 9728
+    g = torch.Generator().manual_seed(5)
+    nw = (1 + 0.1 * torch.randn(H, generator=g)).to(dtype).to(dev)
+    w_gu = (torch.randn(2 * I, H, generator=g) * 0.04).to(dtype).to(dev)
+    w_dn = (torch.randn(H, I, generator=g) * 0.03).to(dtype).to(dev)
+    shared = MlpRowsWorkspace(H, I, dev)
+    for step, (M, with_norm) in enumerate([(8, True), (8, True), (2, True), (8, True), (1, False), (1, True),
+                                           (16, True), (3, False), (2, True), (2, True), (16, True)]):
+        res = torch.randn(1, M, H, generator=g).to(dtype).to(dev)
+        if with_norm:
+            o = _o_partials(M, H, dtype, dev, g)
+            run = lambda ws: add_rmsnorm_mlp_rows(o, res, nw, 1e-6, w_gu, w_dn, ws)
+        else:
+            run = lambda ws: (None, mlp_rows(res, w_gu, w_dn, ws))
+        x_a, d_a = run(shared)
+        fresh = MlpRowsWorkspace(H, I, dev)
+        x_b, d_b = run(fresh)
+        torch.cuda.synchronize()
+        assert not shared.failed() and not fresh.failed(), (step, M)
+        if with_norm:
+            assert torch.equal(x_a, x_b), (step, M)
+        pa = d_a.workspace.view(torch.float32).view(d_a.ksplit, 16, H)[:, :M]
+        pb = d_b.workspace.view(torch.float32).view(d_b.ksplit, 16, H)[:, :M]
+        assert torch.equal(pa, pb), (step, M, (pa - pb).abs().max().item())
+
+
+@pytest.mark.gpu
+def test_gpu_mlp_rows_bounded_wait_gives_up_and_recovers():
+    """The give-up path, forced from the host: the word that holds the number of past launches is set
+    far ahead, so the count that the down workgroups wait for cannot be reached.  The first of them to
+    exhaust its bounded wait (about a second) sets the status word, the others see it and leave, the
+    launch ends normally.  `failed()` then reports it and zeroes the workspace, and the next launch on
+    it equals a launch on a fresh workspace bit for bit."""
+    from ksa_amd import _lib
+    from ksa_amd.gemm import MlpRowsWorkspace, mlp_rows
+    dtype, dev = torch.bfloat16, torch.device("cuda")
+    M, H, I = 8, 2560, 9728
+    g = torch.Generator().manual_seed(9)
+    h = torch.randn(1, M, H, generator=g).to(dtype).to(dev)
+    w_gu = (torch.randn(2 * I, H, generator=g) * 0.04).to(dtype).to(dev)
+    w_dn = (torch.randn(H, I, generator=g) * 0.03).to(dtype).to(dev)
+    ws = MlpRowsWorkspace(H, I, dev)
+    assert _lib.lib().ksa_mlp_rows_status_offset() == 2 * 512
+    ws.buf[:8].view(torch.int64).fill_(1 << 40)   # word 0: launches so far
+    torch.cuda.synchronize()
+    mlp_rows(h, w_gu, w_dn, ws)
+    torch.cuda.synchronize()                       # every workgroup has left
+    assert int(ws._status.item()) == 1
+    assert ws.failed()
+    assert int(ws.buf.view(torch.int64).abs().sum().item()) == 0
+    assert not ws.failed()
+    got = mlp_rows(h, w_gu, w_dn, ws)
+    want = mlp_rows(h, w_gu, w_dn, MlpRowsWorkspace(H, I, dev))
+    torch.cuda.synchronize()
+    assert not ws.failed()
+    assert torch.equal(got.workspace.view(torch.float32).view(got.ksplit, 16, H)[:, :M],
+                       want.workspace.view(torch.float32).view(want.ksplit, 16, H)[:, :M])

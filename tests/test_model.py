@@ -385,3 +385,68 @@ def test_gpu_module_fp16():
         assert log_g.dtype == torch.float32 and gpu.dtype == torch.float16
         rel, agree, _ = _check_logits_and_tokens(log_g.cpu(), log_c, 3e-3, what)
         print(f"fp16 {what}: max logit error {rel:.3e} of the logit scale, arg-max agreement {agree:.2f}")
+
+
+def _mlp_rows_config():
+    """A small decoder whose MLP shape the one-launch MLP kernel takes (hidden size a multiple of 128)."""
+    return tiny_config(summary_chunk_size=128, summary_token_num=8, head_dim=128, num_attention_heads=8,
+                       num_key_value_heads=2, hidden_size=256, intermediate_size=512, num_hidden_layers=3,
+                       summary_sliding_chunk_num=[1, 1 << 20, 1], vocab_size=1000, summary_token_begin=1000)
+
+
+@pytest.mark.gpu
+def test_gpu_one_model_serves_changing_batch_sizes():
+    """Batch 8, then 2, then 8, then 1 on ONE model (one operator set, hence one workspace of the
+    one-launch MLP, whose counting words go on from call to call): every call's logits equal, bit
+    for bit, those of a model made fresh for that call."""
+    from ksa_amd.model import HipOps
+    cfg = _mlp_rows_config()
+    w = init_weights(cfg, "cuda", torch.bfloat16, 31)
+    shared = KsaQwen3ForCausalLM(cfg, w, HipOps())
+    for i, (batch, graph) in enumerate([(8, True), (2, True), (8, False), (1, True), (2, False), (8, True)]):
+        ids = torch.randint(0, cfg.vocab_size, (batch, 140), generator=torch.Generator().manual_seed(40 + i))
+        out_a, log_a = shared.generate(ids, 12, return_logits=True, use_graph=graph)
+        fresh = KsaQwen3ForCausalLM(cfg, w, HipOps())
+        out_b, log_b = fresh.generate(ids, 12, return_logits=True, use_graph=graph)
+        assert shared.ops.mlp_one_launch and fresh.ops.mlp_one_launch
+        assert torch.equal(out_a, out_b), (i, batch)
+        assert torch.equal(log_a, log_b), (i, batch, (log_a - log_b).abs().max().item())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("graph", [False, True])
+def test_gpu_generate_repeats_on_separate_launches_after_a_timeout(graph):
+    """The one-launch MLP's give-up path through the model, forced from the host (the workspace word
+    with the number of past launches is set far ahead, so its waits cannot be satisfied; every
+    workgroup leaves through its bounded wait).  `generate` must notice at its check, switch the
+    operator set to the separate launches, repeat the call, and return what a model that never used
+    the one-launch MLP returns, bit for bit; the steps in between must not have raised or hung.
+    A direct caller of the step functions gets the exception at the next chunk boundary."""
+    from ksa_amd.gemm import MlpRowsTimeout
+    from ksa_amd.model import HipOps
+    cfg = _mlp_rows_config()
+    w = init_weights(cfg, "cuda", torch.bfloat16, 33)
+    ids = torch.randint(0, cfg.vocab_size, (2, 250), generator=torch.Generator().manual_seed(34))
+    plain_ops = HipOps()
+    plain_ops.mlp_one_launch = False
+    want_ids, want_log = KsaQwen3ForCausalLM(cfg, w, plain_ops).generate(ids, 10, return_logits=True, use_graph=graph)
+
+    model = KsaQwen3ForCausalLM(cfg, w, HipOps())
+    ws = model.ops.prepare_mlp_rows(cfg.hidden_size, cfg.intermediate_size, model.device)
+    ws.buf[:8].view(torch.int64).fill_(1 << 40)
+    got_ids, got_log = model.generate(ids, 10, return_logits=True, use_graph=graph)
+    assert not model.ops.mlp_one_launch
+    assert torch.equal(got_ids, want_ids) and torch.equal(got_log, want_log)
+    assert not model.ops.mlp_rows_failed()          # the workspace was cleared
+
+    # the step functions themselves: 250 = 128 + 122, so the sixth step is a chunk boundary
+    model2 = KsaQwen3ForCausalLM(cfg, w, HipOps())
+    logits, cache = model2.prefill(ids)
+    model2.ops.prepare_mlp_rows(cfg.hidden_size, cfg.intermediate_size, model2.device).buf[:8].view(
+        torch.int64).fill_(1 << 40)
+    step = model2.decode_step_graph if graph else model2.decode_step
+    with pytest.raises(MlpRowsTimeout):
+        for _ in range(6):
+            logits = step(logits[:, 0].argmax(-1)[:, None], cache)
+    assert cache.get_cur_chunk_size() == cfg.summary_chunk_size - 1   # raised in front of the boundary step
+    assert not model2.ops.mlp_one_launch
