@@ -409,10 +409,50 @@ def main():
         # library set-up (GEMM handles, index cache, every kernel of the decode path loaded once)
         model.generate(ids[:, :300], 4, use_graph=bool(args.e2e_graph))
         torch.cuda.synchronize()
+        # the cache hand-off inside the prefill, timed with events on the launch stream
+        reorg_ev = []
+        cache_cls = model.ops.cache_cls
+
+        class TimedCache(cache_cls):
+            def reorganize_after_prefill(self, summary_mask):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                super().reorganize_after_prefill(summary_mask)
+                e1.record()
+                reorg_ev.append((e0, e1))
+        model.ops.cache_cls = TimedCache
         t0 = time.perf_counter()
         logits, cache = model.prefill(ids)
         torch.cuda.synchronize()
         t_prefill = time.perf_counter() - t0
+        model.ops.cache_cls = cache_cls
+        reorganize_ms = reorg_ev[-1][0].elapsed_time(reorg_ev[-1][1])
+
+        # Untimed check of what is about to be timed: eight steps launched eagerly and the same eight
+        # replayed from the graph, each on a copy of the cache as the prefill left it, teacher-forced
+        # with the eager run's tokens; the logits must agree within 1 % of the logit scale.
+        import copy
+        n_chk = 8 if args.e2e_graph else 0
+        chk_err = None
+        if n_chk:
+            first = logits.clone()
+            c_e = copy.deepcopy(cache)
+            toks, ref, lg = [], [], first
+            for _ in range(n_chk):
+                toks.append(model.ops.argmax(lg[:, 0])[:, None])
+                lg = model.decode_step(toks[-1], c_e)
+                ref.append(lg[:, 0].float())
+            del c_e
+            c_g = copy.deepcopy(cache)
+            chk_err = 0.0
+            for t in range(n_chk):
+                lg = model.decode_step_graph(toks[t], c_g)
+                scale_ = ref[t].abs().max().item()
+                chk_err = max(chk_err, (lg[:, 0].float() - ref[t]).abs().max().item() / scale_)
+            del c_g, ref, toks, lg
+            torch.cuda.empty_cache()
+            assert chk_err <= 1e-2, f"graph decode differs from eager decode by {chk_err} of the logit scale"
+            logits = first
 
         def attended_rows():   # cache rows one decode step reads, summed over the layers
             return sum(e - a for a, e in (cache.attention_range(li) for li in range(nl)))
@@ -422,25 +462,46 @@ def main():
             return (n + model.lm_head.numel() + weights["norm"].numel()) * 2
 
         rows_first = attended_rows()
+        torch.cuda.synchronize()
         t0 = time.perf_counter()
         n_boundary = 0
+        b_ev = []
         for _ in range(args.e2e_new):
             nxt = model.ops.argmax(logits[:, 0])[:, None]
-            n_boundary += cache.get_cur_chunk_size() == cfg.summary_chunk_size - 1
+            is_b = cache.get_cur_chunk_size() == cfg.summary_chunk_size - 1
+            n_boundary += is_b
+            if is_b:
+                b_ev.append((torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)))
+                b_ev[-1][0].record()
             logits = model.decode_step_graph(nxt, cache) if args.e2e_graph else model.decode_step(nxt, cache)
+            if is_b:
+                b_ev[-1][1].record()
         torch.cuda.synchronize()
         t_decode = time.perf_counter() - t0
+        # pass / fail of the timed run (outside the timed region): no launch gave up waiting, the
+        # last logits are finite, the cache counted every token
+        model.check_steps(cache)
+        assert bool(torch.isfinite(logits.float()).all()), "non-finite logits at the end of the decode run"
+        assert cache.get_true_token_num() == args.e2e_prompt + args.e2e_new
         rows_mean = (rows_first + attended_rows()) / 2
         step_bytes = matrix_bytes() + 2 * rows_mean * cfg.num_key_value_heads * cfg.head_dim * 2 * args.e2e_batch
         floor_ms = step_bytes / (PEAK_HBM_GBPS * 1e9) * 1e3
+        b_ms = [a.elapsed_time(b) for a, b in b_ev]
+        t_in_chunk = t_decode * 1e3 - sum(b_ms)
         result["e2e"] = {
             "workload": f"random-init decoder, {nl} layers (3 Summary W={W} : 1 unbounded window), hidden "
                         f"{cfg.hidden_size}, {Hq}/{Hkv} heads, batch {args.e2e_batch}, prompt "
                         f"{args.e2e_prompt}, {args.e2e_new} greedy steps",
+            "checked": True,
+            "check": {"graph_vs_eager_steps": n_chk, "graph_vs_eager_max_rel_logit_diff": chk_err,
+                      "logits_finite": True, "mlp_one_launch_timeouts": 0},
             "prefill_s": t_prefill, "prefill_tokens_per_s": args.e2e_batch * args.e2e_prompt / t_prefill,
+            "reorganize_ms": reorganize_ms,
             "decode_s": t_decode, "decode_ms_per_step": t_decode / args.e2e_new * 1e3,
             "decode_tokens_per_s": args.e2e_batch * args.e2e_new / t_decode,
-            "chunk_boundary_steps": int(n_boundary), "decode_hip_graph": bool(args.e2e_graph),
+            "chunk_boundary_steps": int(n_boundary), "boundary_step_ms": (sum(b_ms) / len(b_ms)) if b_ms else None,
+            "in_chunk_step_ms": t_in_chunk / max(1, args.e2e_new - len(b_ms)),
+            "decode_hip_graph": bool(args.e2e_graph),
             "decode_step_bytes": int(step_bytes), "decode_hbm_floor_ms": floor_ms,
             "decode_frac_of_hbm_floor": floor_ms / (t_decode / args.e2e_new * 1e3),
             "hbm_allocated_gb": torch.cuda.max_memory_allocated() / 1e9,
@@ -477,7 +538,19 @@ def main():
                     result[key]["roofline"]["traffic"] = t.get(key + "_bytes_per_launch")
         except Exception:
             pass
+    _mark_traffic_source(result)
     print(json.dumps(result))
+
+
+def _mark_traffic_source(result):
+    """Every `roofline.traffic` that is set gets its provenance next to it: these are not read in this
+    run but taken from a separate counter run whose summary is committed."""
+    src = "profiles/hbm_traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, separate run on another box)"
+    recs = [result] + [result[k] for k in ("decode", "pre_attention", "prefill_cfg0", "prefill_cfg1") if k in result]
+    for r in recs:
+        rf = r.get("roofline")
+        if rf is not None and rf.get("traffic") is not None:
+            rf["traffic_source"] = src
 
 
 if __name__ == "__main__":

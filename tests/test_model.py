@@ -450,3 +450,56 @@ def test_gpu_generate_repeats_on_separate_launches_after_a_timeout(graph):
             logits = step(logits[:, 0].argmax(-1)[:, None], cache)
     assert cache.get_cur_chunk_size() == cfg.summary_chunk_size - 1   # raised in front of the boundary step
     assert not model2.ops.mlp_one_launch
+
+
+@pytest.mark.gpu
+def test_gpu_config4_full_depth_decode_equals_prefill():
+    """Config 4 at its own size - 36 layers (three Summary layers with a window of 4 chunks to one
+    unbounded layer, nine times), hidden 2560, 32 / 8 heads, MLP 9728, vocabulary 151936, batch 8,
+    a prompt of 32k tokens: the logits for token n from `prefill(n tokens)` against those from
+    `prefill(n - 9 tokens)` followed by 9 decode steps replayed from the HIP graphs, across the chunk
+    boundary at 32768 tokens (the boundary step runs from its own recording).  The summaries that the
+    boundary step stores are not visible to the text tokens of the next four chunks, so the two ways
+    agree to rounding although the reference's boundary step treats the summary tokens differently
+    from its prefill mask.  This is the decode == prefill invariant through prefill, cache
+    reorganisation (256 chunks, nine text-only gathers of 32k rows), ring, boundary flush and the
+    one-launch MLP at the depth and the size the benchmark's end-to-end run has.
+    Tolerance: both sides are bf16 runs whose rounding errors differ (library GEMMs over 34k rows on one
+    side, the few-rows kernels on the other; different summation orders in attention) and add up over
+    nine times the depth of `test_gpu_module_config4_layer_shape`, i.e. about three times its noise:
+    root mean square within 1 % of the logit scale (measured 0.56 %), largest of the 1.2 million
+    differences within 5 % (measured 2.8 %).  A stale or misplaced cache row in one layer moves the
+    logits by less than that; those are pinned row by row in tests/test_cache_gpu.py.  What this test
+    catches is a step that went wrong as a whole at full depth: garbage or non-finite rows, a layer
+    kind taking the wrong range, a timed-out launch."""
+    from ksa_amd.model import HipOps
+    cfg = KsaQwen3Config()
+    assert cfg.num_hidden_layers == 36 and cfg.sliding_chunk_nums()[:4] == [4, 4, 4, 1 << 20]
+    dev = torch.device("cuda")
+    w = init_weights(cfg, dev, torch.bfloat16, 17)
+    model = KsaQwen3ForCausalLM(cfg, w, HipOps())
+    model.BOUNDARY_GRAPH_AFTER = 0
+    batch, n, k = 8, 32768 + 5, 9
+    ids = torch.randint(0, cfg.vocab_size, (batch, n), generator=torch.Generator().manual_seed(18)).to(dev)
+    want, cache_full = model.prefill(ids)
+    want = want[:, 0].float()
+    assert cache_full.get_true_token_num() == n and cache_full.get_cur_chunk_size() == 5
+    del cache_full
+    torch.cuda.empty_cache()
+    logits, cache = model.prefill(ids[:, :n - k])
+    boundaries = 0
+    for t in range(n - k, n):
+        boundaries += cache.get_cur_chunk_size() == cfg.summary_chunk_size - 1
+        logits = model.decode_step_graph(ids[:, t:t + 1], cache)
+    got = logits[:, 0].float()
+    model.check_steps(cache)                 # raises if a launch gave up waiting
+    assert boundaries == 1 and cache.get_true_token_num() == n
+    assert model.ops.mlp_one_launch
+    assert torch.isfinite(got).all() and torch.isfinite(want).all()
+    scale = want.abs().max().item()
+    err = (got - want).abs().max().item()
+    rms = (got - want).pow(2).mean().sqrt().item()
+    agree = (got.argmax(-1) == want.argmax(-1)).float().mean().item()
+    print(f"full depth: max logit difference {err / scale:.3e} of the logit scale, rms {rms / scale:.3e}, "
+          f"arg-max agreement {agree:.2f}")
+    assert err <= 5e-2 * scale and rms <= 1e-2 * scale, (err / scale, rms / scale)

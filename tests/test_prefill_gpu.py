@@ -261,6 +261,32 @@ def test_prefill_cfg2_sampled_rows():
     assert np.abs(lse[:, rows] - wlse).max() <= 2e-3
 
 
+def test_prefill_dense_causal_layer_batch8_sampled_rows():
+    """The launch an unbounded-window ("full attention") layer of the end-to-end prefill makes: batch 8,
+    34816 expanded rows (32k text), 32 / 8 heads, window larger than the sequence, so every text row
+    sees all earlier text and no summary, and 97 % of the listed tiles are masked ones.  Sequences 0, 3
+    and 7 of the batch (different data each) against the oracle on the first and last chunk's rows,
+    chunk-edge offsets of 16 random chunks and 256 random rows."""
+    import ksa_amd
+    dev = torch.device("cuda")
+    Sq, Hq, Hkv, D, C, S, W, bsz = 34816, 32, 8, 128, 128, 8, 1 << 20, 8
+    B = C + S
+    sp = O.summary_positions(Sq, C, S)
+    qkv = [make_qkv(Sq, Hq, Hkv, D, seed=50 + b) for b in range(bsz)]
+    q, k, v = (torch.stack([t[i] for t in qkv]).to(dev) for i in range(3))
+    out, _ = ksa_amd.summary_attn_func(q, k, v, C, S, W, summary_pos=torch.as_tensor(sp, device=dev))
+    rng = np.random.default_rng(5)
+    rows = set(range(0, B)) | set(range(Sq - B, Sq))
+    for c in rng.choice(Sq // B, 16, replace=False):
+        rows |= {c * B, c * B + C - 1, c * B + C, c * B + B - 1}
+    rows |= set(rng.choice(Sq, 256, replace=False).tolist())
+    rows = np.array(sorted(rows), np.int32)
+    for b in (0, 3, 7):
+        want, _ = c_oracle.attention_rows(to_np(qkv[b][0]), to_np(qkv[b][1]), to_np(qkv[b][2]), C, S, W,
+                                          summary_pos=sp, rows=rows)
+        _compare(to_np(out[b])[rows], want, f"dense causal, sequence {b}")
+
+
 def test_prefill_work_queues_equal_fixed_split():
     """A long launch (32 workgroups per CU and more) hands out its last work items from per-XCD
     queues; a short one gives workgroup i item i.  Three copies of a 32k-row sequence in one batch
