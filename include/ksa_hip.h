@@ -15,7 +15,9 @@
  *   - `stream` is a hipStream_t passed as void* (0 = the null stream);
  *   - 16-bit tensors are described by element strides; pointers must be 16-byte
  *     aligned and strides multiples of 8 elements, the innermost (head_dim) stride is 1;
- *   - dtype: 0 = bf16, 1 = fp16; head_dim 64 or 128;
+ *   - dtype: 0 = bf16, 1 = fp16; head_dim 64, 128 or 256 for the two attention entry points
+ *     (any other multiple of 8 up to 256, which the reference also takes, is zero-padded to the
+ *     next of these by the caller: the Python mirrors do), 64 or 128 for ksa_pre_attention;
  *   - return value 0 = launched, negative = rejected before any launch
  *     (see ksa_error_string).
  */

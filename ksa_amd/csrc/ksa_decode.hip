@@ -50,7 +50,7 @@ constexpr int kWaves = 4;
 constexpr int kRows = 32;  // key rows per wave tile
 
 template <typename T, int D>
-__global__ __launch_bounds__(kThreads, 2) void ksa_decode_kernel(const DecodeParams p) {
+__global__ __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) void ksa_decode_kernel(const DecodeParams p) {
     using Ops = KsaOps<T>;
     constexpr int KS = D / 16;
     constexpr int DB = D / 32;
@@ -376,9 +376,11 @@ int decode_fwd_impl(const void* q, const void* kcache, const void* vcache, void*
     if (dtype == KSA_DTYPE_BF16) {
         if (D == 128) return launch<KsaBf16, 128>(p, batch, st);
         if (D == 64) return launch<KsaBf16, 64>(p, batch, st);
+        if (D == 256) return launch<KsaBf16, 256>(p, batch, st);
     } else {
         if (D == 128) return launch<KsaF16, 128>(p, batch, st);
         if (D == 64) return launch<KsaF16, 64>(p, batch, st);
+        if (D == 256) return launch<KsaF16, 256>(p, batch, st);
     }
     return KSA_ERR_UNSUPPORTED;
 }

@@ -45,6 +45,13 @@
 #include "ksa_mask.h"
 #include "ksa_tile.h"
 
+// This source is compiled as three translation units, so that the instantiations of the kernel
+// compile side by side: unit 0 holds head_dim 64 and 128 and the entry point, units 1 and 2 (which
+// include this file with KSA_PREFILL_UNIT set) the bf16 and the fp16 kernels of head_dim 256.
+#ifndef KSA_PREFILL_UNIT
+#define KSA_PREFILL_UNIT 0
+#endif
+
 namespace {
 
 struct PrefillParams {
@@ -138,7 +145,7 @@ struct PrefillShape {
 };
 
 template <typename T, int D, bool kRegular, int RB, int HW>
-__global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)) void ksa_prefill_kernel(
+__global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 && D <= 128 ? 2 : 1)) void ksa_prefill_kernel(
     const PrefillParams p) {
     constexpr int kThreads = PrefillShape<RB, HW>::kThreads;
     using Ops = KsaOps<T>;
@@ -223,10 +230,14 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
     const char* vbase = reinterpret_cast<const char*>(p.v + bz * p.kv_bs + kvh * p.kv_hs);
     const uint32_t rb = (uint32_t)p.kv_rs * 2u;  // row pitch in bytes
     const int ld_row = tid / CPR;                // first tile row this thread loads
-    auto ksw = [](int r) { return D == 128 ? (r & 15) : ((r >> 1) & 7); };
-    auto vsw = [](int r) { return D == 128 ? (r & 3) : ((r >> 1) & 1); };
+    auto ksw = [](int r) { return D >= 128 ? (r & 15) : ((r >> 1) & 7); };
+    auto vsw = [](int r) { return D >= 128 ? (r & 3) : ((r >> 1) & 1); };
     // this thread fills chunk position tid % CPR of its rows: the source chunk is the position
-    // with the row's permutation undone (rows of one thread differ by multiples of 16 or 32)
+    // with the row's permutation undone.  Rows of one thread differ by multiples of RSTEP: 16 or 32
+    // (the permutation is then the same for all of them), or 8 at head_dim 256, where K's permutation
+    // of a thread's odd loads differs in bit 3 of the chunk number (kKOdd, in bytes).
+    constexpr uint32_t kKOdd = (D >= 128 && RSTEP % 16 != 0) ? 128u : 0u;
+    static_assert(RSTEP % 8 == 0, "a thread's rows differ by multiples of eight");
     const uint32_t kcol = (uint32_t)((tid % CPR) ^ ksw(ld_row)) * 16u;
     const uint32_t vcol = (uint32_t)((tid % CPR) ^ (vsw(ld_row) << 2)) * 16u;
     const uint32_t thr_main = (uint32_t)ld_row * rb;
@@ -275,7 +286,7 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
     };
     // one 1 KB piece (load i of KLD) of tile n into an LDS tile; `col` = kcol or vcol
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-    auto fill1 = [&](const char* base, uint16_t* tile, uint32_t col, int n, uint32_t word, int i) {
+    auto fill1 = [&](const char* base, uint16_t* tile, uint32_t col, int n, uint32_t word, int i, uint32_t odd_xor) {
         uint32_t ub, us, vo[KLD];
         if constexpr (kRegular) {
             const bool in_main = word & 1u;
@@ -294,9 +305,16 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
         // assembly so that the compiler does not track the fill: it would otherwise make LDS
         // reads wait for fills it cannot tell apart; which fills must have landed before a
         // barrier is decided by fills_done.
-        const uint64_t ubase = reinterpret_cast<uint64_t>(base + (ub + us * i));
-        const uint32_t loff = vo[i] + col;
-        const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr)dst;
+        uint64_t ubase = reinterpret_cast<uint64_t>(base + (ub + us * i));
+        const uint32_t loff = vo[i] + (col ^ ((i & 1) ? odd_xor : 0u));
+        uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr)dst;
+        if constexpr (D > 128) {
+            // (both are the same in every lane; at this size the compiler no longer proves it and
+            // would hand the statement below vector registers)
+            lds_addr = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_addr);
+            ubase = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)ubase) |
+                    ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(ubase >> 32)) << 32);
+        }
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm"  // M0 is reserved; nothing else in this kernel uses it
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
@@ -305,9 +323,9 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
                      : "memory", "m0");
 #pragma clang diagnostic pop
     };
-    auto fill = [&](const char* base, uint16_t* tile, uint32_t col, int n, uint32_t word) {
+    auto fill = [&](const char* base, uint16_t* tile, uint32_t col, int n, uint32_t word, uint32_t odd_xor) {
 #pragma unroll
-        for (int i = 0; i < KLD; ++i) fill1(base, tile, col, n, word, i);
+        for (int i = 0; i < KLD; ++i) fill1(base, tile, col, n, word, i, odd_xor);
     };
     // all of this wave's fills have landed (the barrier that follows publishes them)
     auto fills_done = []() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
@@ -617,9 +635,10 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
         // Score MFMAs of the NEXT tile with the probability pairs of THIS tile between them.
         // The fences pin the order; kLead slots run first and cover the first operand reads.
         // The first slots also issue the fills of the two buffers freed by the barrier.
-        constexpr int CPM = 16 / NQK;            // probability pairs per score MFMA
         constexpr int kLead = 3;
-        constexpr int NM = NQK * RB;
+        constexpr int NM = NQK * RB;             // score MFMAs of the step; MFMA m is followed by the
+                                                 // probability slots kLead + [m NCH / NM, (m + 1) NCH / NM)
+                                                 // (two, one, or one at every second MFMA for head_dim 64, 128, 256)
         static_assert(2 * KLD <= NM, "one fill per MFMA slot at most");
 #pragma unroll
         for (int vt = 0; vt < kLead; ++vt) prob_slot(vt);
@@ -639,9 +658,9 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
                     fq[j % kQueue] = (j + kQueue < NQK) ? kfrag(j + kQueue) : vfrag(j + kQueue - NQK);
                 const int m = j * RB + r;
 #pragma unroll
-                for (int vt = kLead + m * CPM; vt < kLead + (m + 1) * CPM; ++vt) prob_slot(vt);
-                if (m < KLD) fill1(kbase, kdst, kcol, nk, wk, m);
-                else if (m < 2 * KLD) fill1(vbase, vdst, vcol, nv, wv, m - KLD);
+                for (int vt = kLead + (m * NCH) / NM; vt < kLead + ((m + 1) * NCH) / NM; ++vt) prob_slot(vt);
+                if (m < KLD) fill1(kbase, kdst, kcol, nk, wk, m, kKOdd);
+                else if (m < 2 * KLD) fill1(vbase, vdst, vcol, nv, wv, m - KLD, 0u);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -721,9 +740,9 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 ? 2 : 1)
         }
         if (ntiles > 0) {  // prologue: K(0), V(0), K(1) in LDS, scores of tile 0
             const int i1 = min(1, ntiles - 1);
-            fill(kbase, Ks0, kcol, seq(0, 0), seq_word(0, 0));
-            fill(vbase, Vs0, vcol, seq(0, 0), seq_word(0, 0));
-            fill(kbase, Ks1, kcol, seq(i1, 0), seq_word(i1, 0));
+            fill(kbase, Ks0, kcol, seq(0, 0), seq_word(0, 0), kKOdd);
+            fill(vbase, Vs0, vcol, seq(0, 0), seq_word(0, 0), 0u);
+            fill(kbase, Ks1, kcol, seq(i1, 0), seq_word(i1, 0), kKOdd);
             fills_done();
             __syncthreads();
             scores(s0, Ks0);
@@ -876,10 +895,25 @@ int launch(const PrefillParams& p, int batch, hipStream_t stream) {
     return launch_shape<T, D, 1, 1>(p, batch, stream);
 }
 
+#if KSA_PREFILL_UNIT == 0
 bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; }
 bool stride_ok(int64_t s) { return (s % 8) == 0; }
+#endif
 
 }  // namespace
+
+#if KSA_PREFILL_UNIT == 1
+int ksa_prefill_launch_d256_bf16(const void* params, int batch, void* stream) {
+    return launch<KsaBf16, 256>(*static_cast<const PrefillParams*>(params), batch, (hipStream_t)stream);
+}
+#elif KSA_PREFILL_UNIT == 2
+int ksa_prefill_launch_d256_f16(const void* params, int batch, void* stream) {
+    return launch<KsaF16, 256>(*static_cast<const PrefillParams*>(params), batch, (hipStream_t)stream);
+}
+#else
+// head_dim 256, in the other two translation units of this source (they see the same PrefillParams)
+int ksa_prefill_launch_d256_bf16(const void* params, int batch, void* stream);
+int ksa_prefill_launch_d256_f16(const void* params, int batch, void* stream);
 
 extern "C" int ksa_prefill_fwd(const void* q, const void* k, const void* v, void* out, float* lse,
                                int batch, int Sq, int Hq, int Hkv, int D, int dtype,
@@ -949,9 +983,12 @@ extern "C" int ksa_prefill_fwd(const void* q, const void* k, const void* v, void
     if (dtype == KSA_DTYPE_BF16) {
         if (D == 128) return launch<KsaBf16, 128>(p, batch, st);
         if (D == 64) return launch<KsaBf16, 64>(p, batch, st);
+        if (D == 256) return ksa_prefill_launch_d256_bf16(&p, batch, stream);
     } else {
         if (D == 128) return launch<KsaF16, 128>(p, batch, st);
         if (D == 64) return launch<KsaF16, 64>(p, batch, st);
+        if (D == 256) return ksa_prefill_launch_d256_f16(&p, batch, stream);
     }
-    return KSA_ERR_UNSUPPORTED;
+    return KSA_ERR_UNSUPPORTED;  // other head dimensions: the caller pads to 64 / 128 / 256
 }
+#endif  // KSA_PREFILL_UNIT

@@ -83,6 +83,22 @@ def ksa_decode(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
         scale = float(D) ** -0.5
     if nsplit is None:
         nsplit = _lib.lib().ksa_decode_auto_splits(b, kcache.shape[1], max_rows)
+    from .prefill import kernel_head_dim, pad_head_dim
+    Dk = kernel_head_dim(D)
+    if Dk != D:
+        # A head dimension without a kernel of its own (the kernels are built for 64 / 128 / 256): the
+        # attended rows are copied into zero-padded buffers for this call.  Correct, but it moves the
+        # rows twice; a cache that stores its rows at a kernel size avoids it.
+        assert D % 8 == 0, "head dimension must be a multiple of 8"
+        if t_start is not None:
+            lo, hi = int(t_start.min().item()), int(t_end.max().item())
+            t_start, t_end = t_start - lo, t_end - lo
+        else:
+            lo, hi, s0, e0 = s0, e0, 0, e0 - s0
+        kcache, vcache = pad_head_dim(kcache[:, :, lo:hi], Dk), pad_head_dim(vcache[:, :, lo:hi], Dk)
+        out = torch.ops.ksa_amd.decode_fwd(pad_head_dim(q, Dk), kcache, vcache, t_start, t_end, s0, e0,
+                                           float(scale), int(nsplit))
+        return out[..., :D].contiguous()
     return torch.ops.ksa_amd.decode_fwd(q, kcache, vcache, t_start, t_end, s0, e0, float(scale), int(nsplit))
 
 

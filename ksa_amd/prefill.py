@@ -150,6 +150,24 @@ def _lastdim_contig(t):
     return t if t.stride(-1) == 1 else t.contiguous()
 
 
+KERNEL_HEAD_DIMS = (64, 128, 256)
+
+
+def kernel_head_dim(D: int) -> int:
+    """The head dimension the kernels run a head dimension D at: the next of 64 / 128 / 256.  The
+    reference takes any multiple of 8 up to 256 (flash_attn/cute/interface.py:206-209); other
+    values are zero-padded to the next kernel size (zero columns add nothing to a score, and the
+    padded output columns are dropped), with the soft-max scale of the true D."""
+    for d in KERNEL_HEAD_DIMS:
+        if D <= d:
+            return d
+    raise AssertionError("head dimension must be at most 256")
+
+
+def pad_head_dim(t: torch.Tensor, Dk: int) -> torch.Tensor:
+    return t if t.shape[-1] == Dk else torch.nn.functional.pad(t, (0, Dk - t.shape[-1]))
+
+
 @torch.library.custom_op("ksa_amd::summary_attn_fwd", mutates_args=())
 def _summary_attn_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
                       mask_cnt: torch.Tensor, mask_idx: torch.Tensor, full_cnt: torch.Tensor,
@@ -239,8 +257,13 @@ def summary_attn_func(q, k, v, chunk_size, summary_num, sliding_chunk_num,
         k = k.contiguous()
     idx = _cached_index(Sq, C, S, W, P, skip_old_summary, q.device)
     scale = float(D) ** -0.5 if softmax_scale is None else float(softmax_scale)
+    Dk = kernel_head_dim(D)
+    if Dk != D:   # a head dimension without a kernel of its own: zero-padded copies (see kernel_head_dim)
+        q, k, v = pad_head_dim(q, Dk), pad_head_dim(k, Dk), pad_head_dim(v, Dk)
     out, lse = torch.ops.ksa_amd.summary_attn_fwd(
         q, k, v, idx[0], idx[1], idx[2], idx[3], C, S, W, P,
         bool(skip_old_summary), phys, scale, bool(return_lse),
         PREFILL_SHAPE if workgroup_shape is None else int(workgroup_shape))
+    if Dk != D:
+        out = out[..., :D].contiguous()
     return out, (lse if return_lse else None)

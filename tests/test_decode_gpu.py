@@ -83,6 +83,18 @@ def test_decode_head_dim_64_and_fp16():
     _check(q, k, v, 3, 555, 1)
 
 
+@pytest.mark.parametrize("D", [256, 96, 192, 40])
+def test_decode_other_head_dims(D):
+    """Head dimension 256 (kernels of its own) and multiples of 8 without one (zero-padded copies of the
+    attended rows at the next kernel size): scalar and per-sequence ranges, splits, the boundary step's
+    9 query tokens, fp16."""
+    q, k, v = _mk(3, 8, 2, 1, D, 900, seed=30 + D)
+    _check(q, k, v, 5, 900, 1)
+    _check(q, k, v, np.array([0, 100, 640], np.int32), np.array([900, 777, 641], np.int32), 3)
+    q, k, v = _mk(2, 4, 2, 9, D, 300, seed=31 + D, dtype=torch.float16)
+    _check(q, k, v, 0, 136, 2)
+
+
 def test_decode_peaked_softmax():
     """large scale -> near one-hot attention: exercises the running-max rescale"""
     q, k, v = _mk(2, 8, 2, 1, 128, 3000, seed=6)

@@ -373,19 +373,48 @@ def test_prefill_rejects_bad_inputs():
     k = torch.zeros(1, 136, 3, 128, device=dev, dtype=torch.bfloat16)
     with pytest.raises(AssertionError):
         ksa_amd.summary_attn_func(q, k, k, 128, 8, 1)
-    q96 = torch.zeros(1, 136, 4, 96, device=dev, dtype=torch.bfloat16)
-    # the reference takes any head_dim <= 256 that is a multiple of 8
-    # (flash_attn/cute/interface.py:206-208); this build has kernels for 64 and 128 only and says so
-    with pytest.raises(ksa_amd.KsaError, match=r"head_dim 64 or 128.*code -3"):
-        ksa_amd.summary_attn_func(q96, q96, q96, 128, 8, 1)
     q264 = torch.zeros(1, 136, 4, 264, device=dev, dtype=torch.bfloat16)
     with pytest.raises(AssertionError, match="at most 256"):   # the reference's own rule
         ksa_amd.summary_attn_func(q264, q264, q264, 128, 8, 1)
-    with pytest.raises(ksa_amd.KsaError, match=r"head_dim 64 or 128.*code -3"):
-        ksa_amd.ksa_decode(q96[:, :1].transpose(1, 2), q96.transpose(1, 2), q96.transpose(1, 2), 0, 136)
+    q100 = torch.zeros(1, 136, 4, 100, device=dev, dtype=torch.bfloat16)
+    with pytest.raises(AssertionError, match="multiple of 8"):
+        ksa_amd.summary_attn_func(q100, q100, q100, 128, 8, 1)
+    # the C layer itself has kernels for 64 / 128 / 256 only and says so (the Python mirror pads)
+    from ksa_amd import _lib
+    q96 = torch.zeros(1, 136, 4, 96, device=dev, dtype=torch.bfloat16)
+    idx = ksa_amd.compute_block_sparsity(136, 136, 128, 8, 1)
+    rc = _lib.lib().ksa_prefill_fwd(q96.data_ptr(), q96.data_ptr(), q96.data_ptr(), q96.data_ptr(), None, 1, 136, 4, 4,
+                                    96, 0, _lib.strides3(q96, (0, 1, 2)), _lib.strides3(q96, (0, 1, 2)),
+                                    _lib.strides3(q96, (0, 1, 2)), 128, 8, 1, 0, 0, 0, idx[0].data_ptr(),
+                                    idx[1].data_ptr(), idx[2].data_ptr(), idx[3].data_ptr(), idx[1].shape[-1], 0.1, 0,
+                                    None, _lib.stream_ptr(dev))
+    assert rc == -3 and b"head_dim 64, 128 or 256" in _lib.lib().ksa_error_string(rc)
     qg = q.clone().requires_grad_(True)
     with pytest.raises(NotImplementedError):
         ksa_amd.summary_attn_func(qg, q, q, 128, 8, 1)
+
+
+@pytest.mark.parametrize("D,dtype", [(256, torch.bfloat16), (256, torch.float16), (96, torch.bfloat16),
+                                     (192, torch.bfloat16), (32, torch.float16), (72, torch.bfloat16)])
+def test_prefill_other_head_dims(D, dtype):
+    """Head dimensions next to 64 / 128: 256 has kernels of its own, any other multiple of 8 up to 256
+    (what the reference takes, flash_attn/cute/interface.py:206-209) runs zero-padded at the next
+    kernel size with the soft-max scale of the true dimension.  Ragged length, GQA, prefix by
+    `summary_pos`, batch 2, lse; against the oracle at the true D."""
+    import ksa_amd
+    dev = torch.device("cuda")
+    Sq, Hq, Hkv, C, S, W = 5 * 136 + 77, 4, 2, 128, 8, 2
+    sp = O.summary_positions(Sq, C, S)
+    qs, ks, vs = zip(*[make_qkv(Sq, Hq, Hkv, D, seed=70 + b, scaled=False) for b in range(2)])
+    q, k, v = (torch.stack(t).to(dtype).to(dev) for t in (qs, ks, vs))
+    out, lse = ksa_amd.summary_attn_func(q, k, v, C, S, W, summary_pos=torch.as_tensor(sp, device=dev),
+                                         return_lse=True)
+    assert out.shape == q.shape and out.dtype == dtype and out.is_contiguous()
+    for b in range(2):
+        want, wlse = c_oracle.attention_rows(to_np(q[b]), to_np(k[b]), to_np(v[b]), C, S, W, summary_pos=sp)
+        tol = ATOL if dtype == torch.bfloat16 else 5e-3
+        assert np.abs(to_np(out[b]) - want).max() <= tol * max(1.0, np.abs(want).max()), (D, b)
+        assert np.abs(to_np(lse[b]) - wlse).max() <= 2e-2 * max(1.0, np.abs(wlse).max())
 
 
 def test_prefill_growing_scores_rebase(wave_rows):
