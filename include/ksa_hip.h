@@ -129,6 +129,23 @@ int ksa_decode_fwd_noalloc(const void* q, const void* kcache, const void* vcache
                            const int64_t* k_strides, const int64_t* v_strides,
                            const int64_t* out_strides, float scale, int nsplit, void* stream);
 
+/* Attention probabilities of a decode step, for callers that ask for them.
+ * Replaces the second result of eager_attention_forward (HF:569-588; selected at HF:643-646 when
+ * config._attn_implementation == "eager"):
+ *   weights = softmax(q K^T * scale (+ mask), fp32).to(dtype)      [batch, Hq, Q, L]
+ * over rows [start_b, end_b) of the cache as in ksa_decode_fwd (whose output the same call site
+ * takes as attn_output); position j of a row is cache row start_b + j, positions past a sequence's
+ * range hold 0, L >= the longest range.  mask: NULL, or additive values of the 16-bit dtype
+ * addressed by mask_strides {batch, head, query token, position} in elements (0 = broadcast).
+ * workspace: ksa_decode_weights_workspace_bytes(batch, Hq, Q, L) bytes (the fp32 scores), 16-byte
+ * aligned.  Two launches; K is read once per kv head. */
+size_t ksa_decode_weights_workspace_bytes(int batch, int Hq, int Q, int L);
+int ksa_decode_weights(const void* q, const void* kcache, void* weights, const void* mask,
+                       const int32_t* start, const int32_t* end, int start0, int end0, int batch, int Hq,
+                       int Hkv, int Q, int D, int dtype, int L, const int64_t* q_strides,
+                       const int64_t* k_strides, const int64_t* mask_strides, float scale, void* workspace,
+                       size_t workspace_bytes, void* stream);
+
 /* Cache row mover.
  * Replaces the Tensor.copy_ sequences of HF:306-336 (update_text), HF:340-398
  * (update_summary), HF:209-302 (reorganize_after_prefill) and the boolean gather of

@@ -11,6 +11,7 @@ express (its cache counters are shared by the batch, :753-754).
 """
 from __future__ import annotations
 
+import ctypes
 from typing import Optional, Tuple
 
 import torch
@@ -100,6 +101,83 @@ def ksa_decode(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
                                            float(scale), int(nsplit))
         return out[..., :D].contiguous()
     return torch.ops.ksa_amd.decode_fwd(q, kcache, vcache, t_start, t_end, s0, e0, float(scale), int(nsplit))
+
+
+def ksa_decode_weights(q: torch.Tensor, kcache: torch.Tensor, start=None, end=None,
+                       scale: Optional[float] = None, mask: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The attention probabilities of `ksa_decode`: softmax(q K^T * scale (+ mask)) over the rows
+    [start, end) of every sequence, computed in fp32 and rounded to q's dtype, [b, Hq, Q, L] with
+    L = the longest range; positions past a shorter sequence's range hold 0.  `mask`, if given, is
+    additive, of q's dtype and broadcastable to [b, Hq, Q, L] (the `attention_mask` of the
+    reference's eager_attention_forward, modeling_qwen3sa.py:569-588)."""
+    assert q.is_cuda and kcache.is_cuda and q.dtype in _DTYPES and q.dtype == kcache.dtype
+    assert q.dim() == 4 and kcache.dim() == 4
+    b, Hq, Q, D = q.shape
+    Hkv, rows = kcache.shape[1], kcache.shape[2]
+    assert kcache.shape[0] == b and kcache.shape[3] == D and Hq % Hkv == 0
+    if q.stride(-1) != 1:
+        q = q.contiguous()
+    assert kcache.stride(-1) == 1, "cache rows must be contiguous"
+    t_start = t_end = None
+    s0, e0 = 0, rows
+    if isinstance(start, torch.Tensor) or isinstance(end, torch.Tensor):
+        t_start = torch.as_tensor(start if start is not None else 0, device=q.device).to(torch.int32).expand(b).contiguous()
+        t_end = torch.as_tensor(end if end is not None else rows, device=q.device).to(torch.int32).expand(b).contiguous()
+        L = int((t_end - t_start).max().item())
+    else:
+        s0 = 0 if start is None else int(start)
+        e0 = rows if end is None else int(end)
+        assert 0 <= s0 < e0 <= rows, "row range out of bounds"
+        L = e0 - s0
+    assert L > 0
+    from .prefill import kernel_head_dim, pad_head_dim
+    Dk = kernel_head_dim(D)
+    if scale is None:
+        scale = float(D) ** -0.5
+    if Dk != D:   # zero-padded copies of the attended rows, as in `ksa_decode`
+        assert D % 8 == 0, "head dimension must be a multiple of 8"
+        if t_start is not None:
+            lo, hi = int(t_start.min().item()), int(t_end.max().item())
+            t_start, t_end = t_start - lo, t_end - lo
+        else:
+            lo, hi, s0, e0 = s0, e0, 0, e0 - s0
+        q, kcache = pad_head_dim(q, Dk), pad_head_dim(kcache[:, :, lo:hi], Dk)
+    m_strides = None
+    if mask is not None:
+        assert mask.dtype == q.dtype and mask.is_cuda
+        mask = mask.expand(b, Hq, Q, L)
+        m_strides = (ctypes.c_int64 * 4)(*mask.stride())
+    lib = _lib.lib()
+    out = torch.empty((b, Hq, Q, L), dtype=q.dtype, device=q.device)
+    ws_bytes = lib.ksa_decode_weights_workspace_bytes(b, Hq, Q, L)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+    with torch.cuda.device(q.device):
+        rc = lib.ksa_decode_weights(
+            q.data_ptr(), kcache.data_ptr(), out.data_ptr(), mask.data_ptr() if mask is not None else None,
+            t_start.data_ptr() if t_start is not None else None, t_end.data_ptr() if t_end is not None else None,
+            s0, e0, b, Hq, Hkv, Q, Dk, _DTYPES[q.dtype], L, _lib.strides3(q, (0, 1, 2)),
+            _lib.strides3(kcache, (0, 1, 2)), m_strides, float(scale), ws.data_ptr(), ws_bytes,
+            _lib.stream_ptr(q.device))
+    _lib.check(rc, "ksa_decode_weights")
+    return out
+
+
+def eager_attention_forward(module, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
+                            attention_mask: Optional[torch.Tensor] = None, scaling: Optional[float] = None,
+                            dropout: float = 0.0, **kwargs) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Drop-in for the reference's `eager_attention_forward` (modeling_qwen3sa.py:569-588), the decode
+    attention function it selects when `config._attn_implementation == "eager"` (:643-646): returns
+    `(attn_output [b, q_len, Hq, D], attn_weights [b, Hq, q_len, L])`.  The output comes from the
+    decode kernel, the probabilities from `ksa_decode_weights` (a second pass over K).  The cache
+    call sites pass no mask (:820-870); one is refused here, because the output kernel has no masked
+    form."""
+    if dropout:
+        raise NotImplementedError("decode attention is inference-only (dropout must be 0)")
+    if attention_mask is not None:
+        raise NotImplementedError("the decode kernels take no attention mask (the reference's cache call sites pass None)")
+    g = query.shape[1] // key.shape[1]
+    assert getattr(module, "num_key_value_groups", g) == g, "module.num_key_value_groups does not match the tensor shapes"
+    return ksa_decode(query, key, value, scale=scaling), ksa_decode_weights(query, key, scale=scaling)
 
 
 def decode_attention_forward(module, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,

@@ -178,3 +178,78 @@ def test_decode_empty_and_single_row_ranges():
         assert np.array_equal(got[1, 0], np.repeat(want1, Hq // Hkv, axis=0))
         ref = c_oracle.decode(q[2:].float().numpy(), kc[2:].float().numpy(), vc[2:].float().numpy(), start[2:], end[2:])
         assert np.abs(got[2:] - ref).max() <= 2e-2
+
+
+def _weights_oracle(q, k, start, end, scale, mask=None):
+    """softmax(q K^T * scale + mask) in float64 per (sequence, head, query token) over rows [start, end)."""
+    Bz, Hq, Q, D = q.shape
+    g = Hq // k.shape[1]
+    L = int(np.max(end - start))
+    out = np.zeros((Bz, Hq, Q, L))
+    for b in range(Bz):
+        n = int(end[b] - start[b])
+        for h in range(Hq):
+            s = q[b, h].astype(np.float64) @ k[b, h // g, start[b]:end[b]].astype(np.float64).T * scale
+            if mask is not None:
+                s = s + np.broadcast_to(mask, (Bz, Hq, Q, L))[b, h, :, :n]
+            s -= s.max(axis=-1, keepdims=True)
+            e = np.exp(s)
+            out[b, h, :, :n] = e / e.sum(axis=-1, keepdims=True)
+    return out
+
+
+@pytest.mark.parametrize("D,dtype", [(128, torch.bfloat16), (64, torch.float16), (256, torch.bfloat16), (96, torch.bfloat16)])
+def test_decode_weights_match_softmax(D, dtype):
+    """The probabilities of the eager decode variant (modeling_qwen3sa.py:569-588) against a float64
+    soft-max of the same scores: per-sequence ranges of different lengths (zeros behind the shorter
+    ones), one query token and the boundary step's nine, GQA, an additive mask; each row sums to 1.
+    Tolerance: the rounding of a probability to the 16-bit type (relative 2^-8 for bf16, 2^-11 for
+    fp16) plus an absolute 1e-6."""
+    import ksa_amd
+    dev = torch.device("cuda")
+    rel = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    for Q, rows, start, end in ((1, 900, np.array([0, 100, 640]), np.array([900, 777, 641])),
+                                (9, 300, np.array([3, 3, 3]), np.array([139, 139, 139]))):
+        q, k, v = _mk(3, 8, 2, Q, D, rows, seed=90 + Q + D, dtype=dtype)
+        scale = D ** -0.5
+        st, en = (torch.as_tensor(x, dtype=torch.int32, device=dev) for x in (start, end))
+        w = ksa_amd.ksa_decode_weights(q.to(dev), k.to(dev), st, en)
+        L = int((end - start).max())
+        assert w.shape == (3, 8, Q, L) and w.dtype == dtype
+        want = _weights_oracle(to_np(q), to_np(k), start, end, scale)
+        got = to_np(w).astype(np.float64)
+        assert (np.abs(got - want) <= rel * want + 1e-6).all(), np.abs(got - want).max()
+        assert np.abs(got.sum(-1) - 1).max() <= 2e-2
+        for b in range(3):
+            assert (got[b, :, :, end[b] - start[b]:] == 0).all()
+    # scalar range + additive mask that removes every third position and biases the rest
+    q, k, v = _mk(2, 4, 4, 2, D, 200, seed=99, dtype=dtype)
+    mask = torch.zeros(2, 1, 2, 150, dtype=dtype)
+    mask[..., ::3] = float("-inf")
+    mask[..., 1::3] = 0.5
+    w = ksa_amd.ksa_decode_weights(q.to(dev), k.to(dev), 20, 170, mask=mask.to(dev))
+    want = _weights_oracle(to_np(q), to_np(k), np.full(2, 20), np.full(2, 170), D ** -0.5, mask=to_np(mask).astype(np.float64))
+    got = to_np(w).astype(np.float64)
+    assert (np.abs(got - want) <= rel * want + 1e-6).all() and (got[..., ::3] == 0).all()
+
+
+def test_eager_attention_forward_signature():
+    """The reference's eager decode attention function (modeling_qwen3sa.py:569-588), as its cache call
+    sites use it (:816-870: a slice of the cache, mask None): output equal to the SDPA variant's,
+    probabilities consistent with it (weights @ V reproduces the output)."""
+    import ksa_amd
+    dev = torch.device("cuda")
+    q, k, v = _mk(2, 8, 2, 1, 128, 500, seed=123)
+    q, k, v = q.to(dev), k.to(dev), v.to(dev)
+
+    class M:
+        num_key_value_groups = 4
+    out, w = ksa_amd.eager_attention_forward(M(), q, k[:, :, 7:444], v[:, :, 7:444], None, scaling=128 ** -0.5)
+    ref, none = ksa_amd.decode_attention_forward(M(), q, k[:, :, 7:444], v[:, :, 7:444], None, scaling=128 ** -0.5)
+    assert none is None and torch.equal(out, ref)
+    assert w.shape == (2, 8, 1, 437)
+    vv = v[:, :, 7:444].float().repeat_interleave(4, dim=1)           # [b, Hq, L, D]
+    recon = torch.matmul(w.float(), vv).transpose(1, 2)                # [b, 1, Hq, D]
+    assert (recon - out.float()).abs().max().item() <= 2e-2
+    with pytest.raises(NotImplementedError):
+        ksa_amd.eager_attention_forward(M(), q, k, v, torch.zeros(1, device=dev), scaling=1.0)
