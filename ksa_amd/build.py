@@ -10,7 +10,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libksa_hip.so")
 # (the slowest units first: they run next to the others)
-SOURCES = ["ksa_prefill_d256_bf16.hip", "ksa_prefill_d256_f16.hip", "ksa_prefill.hip", "ksa_api.hip", "ksa_index.hip", "ksa_decode.hip", "ksa_decode_weights.hip", "ksa_cache.hip",
+SOURCES = ["ksa_prefill_d256_bf16_regular.hip", "ksa_prefill_d256_bf16_general.hip", "ksa_prefill_d256_f16_regular.hip",
+           "ksa_prefill_d256_f16_general.hip", "ksa_prefill.hip", "ksa_api.hip", "ksa_index.hip", "ksa_decode.hip", "ksa_decode_weights.hip", "ksa_cache.hip",
            "ksa_pre.hip", "ksa_elementwise.hip", "ksa_gemm_rows.hip", "ksa_mlp_rows.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",

@@ -45,11 +45,20 @@
 #include "ksa_mask.h"
 #include "ksa_tile.h"
 
-// This source is compiled as three translation units, so that the instantiations of the kernel
-// compile side by side: unit 0 holds head_dim 64 and 128 and the entry point, units 1 and 2 (which
-// include this file with KSA_PREFILL_UNIT set) the bf16 and the fp16 kernels of head_dim 256.
+// This source is compiled as five translation units, so that the instantiations of the kernel
+// compile side by side: unit 0 holds head_dim 64 and 128 and the entry point; units 1 to 4 (files
+// that include this one with KSA_PREFILL_UNIT set) hold one kernel of head_dim 256 each - bf16 /
+// fp16, regular / general tile addressing - because each of those takes over a minute to compile.
 #ifndef KSA_PREFILL_UNIT
 #define KSA_PREFILL_UNIT 0
+#endif
+// which of the two addressing variants a unit instantiates in launch_shape: 0 both, 1 regular, 2 general
+#if KSA_PREFILL_UNIT == 1 || KSA_PREFILL_UNIT == 3
+#define KSA_PREFILL_VARIANTS 1
+#elif KSA_PREFILL_UNIT == 2 || KSA_PREFILL_UNIT == 4
+#define KSA_PREFILL_VARIANTS 2
+#else
+#define KSA_PREFILL_VARIANTS 0
 #endif
 
 namespace {
@@ -852,13 +861,20 @@ __global__ void ksa_prefill_zero_queues_kernel(int32_t* sched) {
     if (threadIdx.x < 8) sched[threadIdx.x] = 0;
 }
 
+// whether a launch can use the kernel variant with regular tile addressing (see kRegular)
+template <int D, int RB, int HW>
+bool prefill_regular(const PrefillParams& p) {
+    constexpr int RSTEP = PrefillShape<RB, HW>::kThreads / (D / 8);
+    const KsaMask& mk = p.mk;
+    const bool prefix_ok = mk.P == 0 || p.phys_prefix || (RSTEP % mk.S == 0 && mk.P % kTileN == 0);
+    return prefix_ok && mk.Sk % kTileN == 0;
+}
+
 template <typename T, int D, int RB, int HW>
 int launch_shape(const PrefillParams& p, int batch, hipStream_t stream) {
     constexpr int kThreads = PrefillShape<RB, HW>::kThreads;
-    constexpr int RSTEP = kThreads / (D / 8);
-    const KsaMask& mk = p.mk;
-    const bool prefix_ok = mk.P == 0 || p.phys_prefix || (RSTEP % mk.S == 0 && mk.P % kTileN == 0);
-    const bool regular = prefix_ok && mk.Sk % kTileN == 0;
+    const bool regular = prefill_regular<D, RB, HW>(p);
+    if ((KSA_PREFILL_VARIANTS == 1 && !regular) || (KSA_PREFILL_VARIANTS == 2 && regular)) return KSA_ERR_INVALID;
     PrefillParams pp = p;
     pp.n_items = p.M * (p.Hq / HW);
     pp.total = pp.n_items * batch;
@@ -876,10 +892,12 @@ int launch_shape(const PrefillParams& p, int batch, hipStream_t stream) {
         pp.sched = nullptr;
     }
     dim3 grid(pp.total + spare);
-    if (regular)
-        hipLaunchKernelGGL((ksa_prefill_kernel<T, D, true, RB, HW>), grid, dim3(kThreads), 0, stream, pp);
-    else
-        hipLaunchKernelGGL((ksa_prefill_kernel<T, D, false, RB, HW>), grid, dim3(kThreads), 0, stream, pp);
+#if KSA_PREFILL_VARIANTS != 2
+    if (regular) hipLaunchKernelGGL((ksa_prefill_kernel<T, D, true, RB, HW>), grid, dim3(kThreads), 0, stream, pp);
+#endif
+#if KSA_PREFILL_VARIANTS != 1
+    if (!regular) hipLaunchKernelGGL((ksa_prefill_kernel<T, D, false, RB, HW>), grid, dim3(kThreads), 0, stream, pp);
+#endif
     return ksa_check_launch();
 }
 
@@ -902,18 +920,28 @@ bool stride_ok(int64_t s) { return (s % 8) == 0; }
 
 }  // namespace
 
+// head_dim 256: one launcher per translation unit (they all see the same PrefillParams)
+int ksa_prefill_launch_d256_bf16_regular(const void* params, int batch, void* stream);
+int ksa_prefill_launch_d256_bf16_general(const void* params, int batch, void* stream);
+int ksa_prefill_launch_d256_f16_regular(const void* params, int batch, void* stream);
+int ksa_prefill_launch_d256_f16_general(const void* params, int batch, void* stream);
 #if KSA_PREFILL_UNIT == 1
-int ksa_prefill_launch_d256_bf16(const void* params, int batch, void* stream) {
+int ksa_prefill_launch_d256_bf16_regular(const void* params, int batch, void* stream) {
     return launch<KsaBf16, 256>(*static_cast<const PrefillParams*>(params), batch, (hipStream_t)stream);
 }
 #elif KSA_PREFILL_UNIT == 2
-int ksa_prefill_launch_d256_f16(const void* params, int batch, void* stream) {
+int ksa_prefill_launch_d256_bf16_general(const void* params, int batch, void* stream) {
+    return launch<KsaBf16, 256>(*static_cast<const PrefillParams*>(params), batch, (hipStream_t)stream);
+}
+#elif KSA_PREFILL_UNIT == 3
+int ksa_prefill_launch_d256_f16_regular(const void* params, int batch, void* stream) {
+    return launch<KsaF16, 256>(*static_cast<const PrefillParams*>(params), batch, (hipStream_t)stream);
+}
+#elif KSA_PREFILL_UNIT == 4
+int ksa_prefill_launch_d256_f16_general(const void* params, int batch, void* stream) {
     return launch<KsaF16, 256>(*static_cast<const PrefillParams*>(params), batch, (hipStream_t)stream);
 }
 #else
-// head_dim 256, in the other two translation units of this source (they see the same PrefillParams)
-int ksa_prefill_launch_d256_bf16(const void* params, int batch, void* stream);
-int ksa_prefill_launch_d256_f16(const void* params, int batch, void* stream);
 
 extern "C" int ksa_prefill_fwd(const void* q, const void* k, const void* v, void* out, float* lse,
                                int batch, int Sq, int Hq, int Hkv, int D, int dtype,
@@ -983,11 +1011,15 @@ extern "C" int ksa_prefill_fwd(const void* q, const void* k, const void* v, void
     if (dtype == KSA_DTYPE_BF16) {
         if (D == 128) return launch<KsaBf16, 128>(p, batch, st);
         if (D == 64) return launch<KsaBf16, 64>(p, batch, st);
-        if (D == 256) return ksa_prefill_launch_d256_bf16(&p, batch, stream);
+        if (D == 256)
+            return prefill_regular<256, 1, 1>(p) ? ksa_prefill_launch_d256_bf16_regular(&p, batch, stream)
+                                                 : ksa_prefill_launch_d256_bf16_general(&p, batch, stream);
     } else {
         if (D == 128) return launch<KsaF16, 128>(p, batch, st);
         if (D == 64) return launch<KsaF16, 64>(p, batch, st);
-        if (D == 256) return ksa_prefill_launch_d256_f16(&p, batch, stream);
+        if (D == 256)
+            return prefill_regular<256, 1, 1>(p) ? ksa_prefill_launch_d256_f16_regular(&p, batch, stream)
+                                                 : ksa_prefill_launch_d256_f16_general(&p, batch, stream);
     }
     return KSA_ERR_UNSUPPORTED;  // other head dimensions: the caller pads to 64 / 128 / 256
 }
