@@ -111,6 +111,21 @@ int ksa_decode_fwd(const void* q, const void* kcache, const void* vcache, void* 
                    const int64_t* k_strides, const int64_t* v_strides, const int64_t* out_strides,
                    float scale, int nsplit, void* workspace, size_t workspace_bytes, void* stream);
 
+/* Chunk-boundary decode step in one launch (HF:831-876, the two calls of the decode attention
+ * function and the torch.cat behind them): query token 0 (the chunk's last text token) attends rows
+ * [text_start, text_end), query tokens 1 .. Q - 1 (its summary tokens) attend [sum_start, sum_end),
+ * both un-masked; each pair of bounds as device int32[batch] or, when NULL, the scalars behind it.
+ * The two groups of columns read their rows separately (the text token's g columns do not ride
+ * through the summary tokens' range and vice versa).  Everything else as ksa_decode_fwd; Q >= 2,
+ * Hq / Hkv <= 32; workspace ksa_decode_boundary_workspace_bytes(...) bytes when nsplit > 1. */
+size_t ksa_decode_boundary_workspace_bytes(int batch, int Hq, int Hkv, int Q, int D, int nsplit);
+int ksa_decode_boundary_fwd(const void* q, const void* kcache, const void* vcache, void* out,
+                            const int32_t* text_start, const int32_t* text_end, int text_start0, int text_end0,
+                            const int32_t* sum_start, const int32_t* sum_end, int sum_start0, int sum_end0,
+                            int batch, int Hq, int Hkv, int Q, int D, int dtype, const int64_t* q_strides,
+                            const int64_t* k_strides, const int64_t* v_strides, const int64_t* out_strides,
+                            float scale, int nsplit, void* workspace, size_t workspace_bytes, void* stream);
+
 /* ksa_decode_fwd for callers that cannot allocate device memory (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
  * Same arguments and results as ksa_decode_fwd without the workspace: the split-K partials go to
@@ -157,6 +172,17 @@ int ksa_copy_rows(const void* src, void* dst, const int32_t* src_index,
                   const int32_t* dst_start_seq, int src_start, int dst_start, int nrows, int batch,
                   int heads, int D, const int64_t* src_strides, const int64_t* dst_strides,
                   void* stream);
+
+/* Up to 8 independent row moves of one shape (same batch, heads, D) as one launch; move m as
+ * ksa_copy_rows without a source index list: dst[m] row (dst_start[m] + i, or dst_start_seq[m][b] + i
+ * when that device array is given) <- src[m] row (src_start[m] + i), i < nrows[m].  src_strides /
+ * dst_strides hold 3 strides {batch, head, row} per move.  No move may read rows that another one
+ * writes.  The moves of a chunk-boundary step (HF:306-336 for its text token, HF:340-398 for the flush
+ * and the append, the scratch-row copies of HF:476-497) are two such launches instead of twelve. */
+int ksa_copy_rows_multi(int n_moves, const void* const* src, void* const* dst,
+                        const int32_t* const* dst_start_seq, const int* src_start, const int* dst_start,
+                        const int* nrows, int batch, int heads, int D, const int64_t* src_strides,
+                        const int64_t* dst_strides, void* stream);
 
 /* Pre-attention step: per-head RMSNorm of q and k, rotary embedding, layout write of q, k, v.
  * Replaces HF:660-666 (q_norm / k_norm = Qwen3RMSNorm HF:64-79 on head_dim, the three

@@ -11,7 +11,8 @@ from ._lib import KsaError, lib as _load
 _load()
 
 from .prefill import SUMMARY_ATTN_CACHE, compute_block_sparsity, summary_attn_func  # noqa: E402
-from .decode import decode_attention_forward, eager_attention_forward, ksa_decode, ksa_decode_weights  # noqa: E402
+from .decode import (decode_attention_forward, eager_attention_forward, ksa_decode, ksa_decode_boundary,  # noqa: E402
+                     ksa_decode_weights)
 from .cache import Qwen3RingBufferCache  # noqa: E402
 from .pre import pre_attention  # noqa: E402
 from .elementwise import add_rmsnorm, silu_mul  # noqa: E402
@@ -20,6 +21,6 @@ from .model import KsaQwen3Config, KsaQwen3ForCausalLM, init_weights  # noqa: E4
 
 __all__ = [
     "KsaError", "SUMMARY_ATTN_CACHE", "compute_block_sparsity", "summary_attn_func",
-    "decode_attention_forward", "eager_attention_forward", "ksa_decode", "ksa_decode_weights", "Qwen3RingBufferCache", "pre_attention", "add_rmsnorm", "silu_mul", "linear_rows",
+    "decode_attention_forward", "eager_attention_forward", "ksa_decode", "ksa_decode_boundary", "ksa_decode_weights", "Qwen3RingBufferCache", "pre_attention", "add_rmsnorm", "silu_mul", "linear_rows",
     "KsaQwen3Config", "KsaQwen3ForCausalLM", "init_weights",
 ]

@@ -32,6 +32,10 @@ _SIGNATURES = {
     "ksa_decode_fwd_noalloc": (_int, [_vp] * 6 + [_int] * 8 + [_i64p] * 4 + [ctypes.c_float, _int, _vp]),
     "ksa_decode_weights_workspace_bytes": (ctypes.c_size_t, [_int] * 4),
     "ksa_decode_weights": (_int, [_vp] * 6 + [_int] * 9 + [_i64p, _i64p, _vp] + [ctypes.c_float, _vp, ctypes.c_size_t, _vp]),
+    "ksa_decode_boundary_workspace_bytes": (ctypes.c_size_t, [_int] * 6),
+    "ksa_decode_boundary_fwd": (_int, [_vp] * 6 + [_int, _int, _vp, _vp] + [_int] * 8 + [_i64p] * 4
+                                + [ctypes.c_float, _int, _vp, ctypes.c_size_t, _vp]),
+    "ksa_copy_rows_multi": (_int, [_int, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp, _vp, _vp]),
     "ksa_copy_rows": (_int, [_vp] * 4 + [_int] * 6 + [_i64p] * 2 + [_vp]),
     "ksa_pre_attention": (_int, [_vp] * 10 + [_int] * 6 + [_i64p] * 7 + [_vp, ctypes.c_float, _vp]),
     "ksa_pre_attention_partials": (_int, [_vp, _int] + [_vp] * 7 + [_int] * 6 + [_i64p] * 4

@@ -49,6 +49,45 @@ def _move_rows(src: torch.Tensor, dst: torch.Tensor, nrows: int, src_start: int 
     _lib.check(rc, "ksa_copy_rows")
 
 
+def _move_rows_multi(moves) -> None:
+    """Up to 8 independent `_move_rows` (without source index lists) as one launch.  Each move is
+    (src, dst, nrows, src_start, dst_start) with dst_start an int or an int32 GPU tensor [bsz] (read
+    at run time); all tensors [bsz, heads, rows, D] of one shape class.  No move may read rows that
+    another one writes."""
+    moves = [m for m in moves if m[2] > 0]
+    if not moves:
+        return
+    import ctypes
+    bsz, heads, _, D = moves[0][1].shape
+    n = len(moves)
+    keep = []
+    srcs, dsts, seqs = (ctypes.c_void_p * n)(), (ctypes.c_void_p * n)(), (ctypes.c_void_p * n)()
+    s0, d0, nr = (ctypes.c_int * n)(), (ctypes.c_int * n)(), (ctypes.c_int * n)()
+    sst, dst_ = (ctypes.c_int64 * (3 * n))(), (ctypes.c_int64 * (3 * n))()
+    for i, (src, dst, nrows, src_start, dst_start) in enumerate(moves):
+        assert src.is_cuda and dst.is_cuda and src.dtype == dst.dtype and src.element_size() == 2
+        assert dst.shape[0] == bsz and dst.shape[1] == heads and dst.shape[3] == D
+        if src.stride(-1) != 1:
+            src = src.contiguous()
+        if src.shape[0] != bsz or src.shape[1] != heads:
+            src = src.expand(bsz, heads, src.shape[2], D)
+        keep.append(src)
+        srcs[i], dsts[i] = src.data_ptr(), dst.data_ptr()
+        if torch.is_tensor(dst_start):
+            assert dst_start.dtype == torch.int32 and dst_start.is_cuda and dst_start.numel() == bsz
+            seqs[i], d0[i] = dst_start.data_ptr(), 0
+        else:
+            seqs[i], d0[i] = None, int(dst_start)
+        s0[i], nr[i] = int(src_start), int(nrows)
+        for j, dim in enumerate((0, 1, 2)):
+            sst[3 * i + j], dst_[3 * i + j] = src.stride(dim), dst.stride(dim)
+    dev = moves[0][1].device
+    with torch.cuda.device(dev):
+        rc = _lib.lib().ksa_copy_rows_multi(n, srcs, dsts, seqs, s0, d0, nr, bsz, heads, D, sst, dst_,
+                                            _lib.stream_ptr(dev))
+    _lib.check(rc, "ksa_copy_rows_multi")
+
+
 class Qwen3RingBufferCache:
     is_compileable = False
     _SUMMARY_INIT_CAP = 512

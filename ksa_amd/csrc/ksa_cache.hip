@@ -41,7 +41,66 @@ __global__ __launch_bounds__(256) void ksa_copy_rows_kernel(const CopyParams p) 
     }
 }
 
+// Several independent row moves of one shape (same batch, heads, head_dim) as one launch: the moves of
+// a chunk-boundary step (text row, summary rows into the scratch rows; afterwards the flush of the
+// chunk into the ring and the append of its summaries, for K and for V) are eight launches otherwise.
+constexpr int kMaxMoves = 8;
+struct MultiCopyParams {
+    CopyParams mv[kMaxMoves];
+};
+
+__global__ __launch_bounds__(256) void ksa_copy_rows_multi_kernel(const MultiCopyParams mp, int heads) {
+    const int which = blockIdx.y / heads, h = blockIdx.y % heads, b = blockIdx.z;
+    const CopyParams& p = mp.mv[which];
+    const int64_t total = (int64_t)p.nrows * p.cpr;
+    const uint16_t* sb = p.src + b * p.s_bs + h * p.s_hs;
+    uint16_t* db = p.dst + b * p.d_bs + h * p.d_hs;
+    const int d0 = p.dst_start_seq ? p.dst_start_seq[b] : p.dst_start;
+    for (int64_t u = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; u < total;
+         u += (int64_t)gridDim.x * blockDim.x) {
+        const int i = (int)(u / p.cpr), c = (int)(u % p.cpr);
+        *reinterpret_cast<u32x4*>(db + (int64_t)(d0 + i) * p.d_rs + 8 * c) =
+            __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(sb + (int64_t)(p.src_start + i) * p.s_rs + 8 * c));
+    }
+}
+
 }  // namespace
+
+// n_moves <= 8 moves, move m: dst[m] row (dst_start[m] (+ dst_start_seq[m][sequence] instead, if given) + i)
+// <- src[m] row (src_start[m] + i), i < nrows[m], for every (sequence, head).  The moves must not
+// depend on each other (no move reads rows that another one writes): they run side by side.
+extern "C" int ksa_copy_rows_multi(int n_moves, const void* const* src, void* const* dst,
+                                   const int32_t* const* dst_start_seq, const int* src_start, const int* dst_start,
+                                   const int* nrows, int batch, int heads, int D, const int64_t* src_strides,
+                                   const int64_t* dst_strides, void* stream) {
+    if (!src || !dst || !src_start || !dst_start || !nrows || !src_strides || !dst_strides) return KSA_ERR_NULL;
+    if (n_moves <= 0 || n_moves > kMaxMoves || batch <= 0 || heads <= 0 || D <= 0 || D % 8 != 0) return KSA_ERR_INVALID;
+    MultiCopyParams mp{};
+    int64_t most = 0;
+    for (int m = 0; m < n_moves; ++m) {
+        if (!src[m] || !dst[m]) return KSA_ERR_NULL;
+        if (nrows[m] < 0 || src_start[m] < 0 || dst_start[m] < 0) return KSA_ERR_INVALID;
+        if ((reinterpret_cast<uintptr_t>(src[m]) | reinterpret_cast<uintptr_t>(dst[m])) & 15) return KSA_ERR_ALIGN;
+        for (int i = 0; i < 3; ++i)
+            if ((src_strides[3 * m + i] % 8) || (dst_strides[3 * m + i] % 8)) return KSA_ERR_ALIGN;
+        CopyParams& p = mp.mv[m];
+        p.src = (const uint16_t*)src[m];
+        p.dst = (uint16_t*)dst[m];
+        p.dst_start_seq = dst_start_seq ? dst_start_seq[m] : nullptr;
+        p.src_start = src_start[m], p.dst_start = dst_start[m], p.nrows = nrows[m];
+        p.cpr = D / 8;
+        p.s_bs = src_strides[3 * m], p.s_hs = src_strides[3 * m + 1], p.s_rs = src_strides[3 * m + 2];
+        p.d_bs = dst_strides[3 * m], p.d_hs = dst_strides[3 * m + 1], p.d_rs = dst_strides[3 * m + 2];
+        const int64_t total = (int64_t)nrows[m] * p.cpr;
+        if (total > most) most = total;
+    }
+    if (most == 0) return KSA_OK;
+    int gx = (int)((most + 255) / 256);
+    if (gx > 1024) gx = 1024;
+    hipLaunchKernelGGL(ksa_copy_rows_multi_kernel, dim3(gx, heads * n_moves, batch), dim3(256), 0, (hipStream_t)stream,
+                       mp, heads);
+    return ksa_check_launch();
+}
 
 extern "C" int ksa_copy_rows(const void* src, void* dst, const int32_t* src_index,
                              const int32_t* dst_start_seq, int src_start, int dst_start, int nrows,

@@ -43,7 +43,35 @@ struct DecodeParams {
     float* ws_ml;  // [B,Hkv,nsplit,ncols_pad,2]  (max in log2 units, sum)
     int ncols_pad;
     float scale_log2;
+    // Chunk-boundary form (split_q != 0): query token 0 (the chunk's last text token) attends the rows
+    // [start, end) and has column block 0 to itself (g columns); the other Q - 1 query tokens (the
+    // chunk's summary tokens) attend [start2, end2) and fill the column blocks behind it.
+    int split_q;
+    const int32_t* start2;
+    const int32_t* end2;
+    int start20, end20;
 };
+
+// column lq of column block colblk -> (query token, head in the group); false: no such column
+__device__ __forceinline__ bool ksa_decode_column(const DecodeParams& p, int colblk, int lq, int& qi, int& gi) {
+    if (!p.split_q) {
+        const int col = colblk * 32 + lq;
+        qi = col / p.g, gi = col % p.g;
+        return col < p.ncols;
+    }
+    if (colblk == 0) {
+        qi = 0, gi = lq;
+        return lq < p.g;
+    }
+    const int c = (colblk - 1) * 32 + lq;
+    qi = 1 + c / p.g, gi = c % p.g;
+    return c < (p.Q - 1) * p.g;
+}
+// slot of the logical column (query token qi, head gi) in the workspace's column axis
+__device__ __forceinline__ int ksa_decode_slot(const DecodeParams& p, int qi, int gi) {
+    if (!p.split_q) return qi * p.g + gi;
+    return qi == 0 ? gi : 32 + (qi - 1) * p.g + gi;
+}
 
 constexpr int kThreads = 256;
 constexpr int kWaves = 4;
@@ -78,8 +106,9 @@ __global__ __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) void ksa_decode_kerne
     uint16_t* Kw = reinterpret_cast<uint16_t*>(smem) + wave * kStage;
     uint16_t* Vw = Kw + kRows * KROW;
 
-    const int r_begin = p.start ? p.start[bz] : p.start0;
-    const int r_end = p.end ? p.end[bz] : p.end0;
+    const bool second = p.split_q && colblk > 0;  // the summary tokens' columns and their own row range
+    const int r_begin = second ? (p.start2 ? p.start2[bz] : p.start20) : (p.start ? p.start[bz] : p.start0);
+    const int r_end = second ? (p.end2 ? p.end2[bz] : p.end20) : (p.end ? p.end[bz] : p.end0);
     const int L = max(r_end - r_begin, 0);
     // rows per split: a multiple of the 128 rows the four waves cover per round
     const int per = ((L + p.nsplit - 1) / p.nsplit + kWaves * kRows - 1) / (kWaves * kRows) *
@@ -88,10 +117,9 @@ __global__ __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) void ksa_decode_kerne
     const int s1 = min(r_end, s0 + per);
 
     // column (query token qi, head gi of the group) owned by this lane
-    const int col = colblk * 32 + lq;
-    const bool col_ok = col < p.ncols;
-    const int qi = col_ok ? col / p.g : 0;
-    const int gi = col_ok ? col % p.g : 0;
+    int qi, gi;
+    const bool col_ok = ksa_decode_column(p, colblk, lq, qi, gi);
+    if (!col_ok) qi = 0, gi = 0;
     const int head = kvh * p.g + gi;
 
     u32x4 qf[KS];
@@ -216,7 +244,8 @@ __global__ __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) void ksa_decode_kerne
         }
     }
     __syncthreads();
-    const int ncol_here = min(32, p.ncols - colblk * 32);
+    const int ncol_here = !p.split_q ? min(32, p.ncols - colblk * 32)
+                                     : (colblk == 0 ? p.g : min(32, (p.Q - 1) * p.g - (colblk - 1) * 32));
     for (int e = tid; e < ncol_here * D; e += kThreads) {
         const int c = e / D, d = e % D;
         float mx = -INFINITY;
@@ -232,7 +261,8 @@ __global__ __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) void ksa_decode_kerne
         }
         const int cg = colblk * 32 + c;
         if (p.nsplit == 1) {
-            const int oq = cg / p.g, og = cg % p.g;
+            int oq, og;
+            ksa_decode_column(p, colblk, c, oq, og);
             const float val = l > 0.f ? acc / l : 0.f;
             uint16_t* op = p.out + bz * p.o_bs + oq * p.o_qs + (kvh * p.g + og) * p.o_hs + d;
             const uint32_t pk = Ops::pack2(val, 0.f);
@@ -252,7 +282,8 @@ __global__ __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) void ksa_decode_kerne
 template <typename T, int D>
 __global__ __launch_bounds__(D) void ksa_decode_merge_kernel(const DecodeParams p) {
     using Ops = KsaOps<T>;
-    const int cg = blockIdx.x;
+    const int oq = blockIdx.x / p.g, og = blockIdx.x % p.g;  // logical column: query token, head in the group
+    const int cg = ksa_decode_slot(p, oq, og);
     const int kvh = blockIdx.y;
     const int bz = blockIdx.z;
     const int d = threadIdx.x;
@@ -285,7 +316,6 @@ __global__ __launch_bounds__(D) void ksa_decode_merge_kernel(const DecodeParams 
             }
         }
     }
-    const int oq = cg / p.g, og = cg % p.g;
     const float val = l > 0.f ? acc / l : 0.f;
     uint16_t* op = p.out + bz * p.o_bs + oq * p.o_qs + (kvh * p.g + og) * p.o_hs + d;
     *op = (uint16_t)(Ops::pack2(val, 0.f) & 0xffffu);
@@ -293,7 +323,7 @@ __global__ __launch_bounds__(D) void ksa_decode_merge_kernel(const DecodeParams 
 
 template <typename T, int D>
 int launch(const DecodeParams& p, int batch, hipStream_t stream) {
-    const int colblks = (p.ncols + 31) / 32;
+    const int colblks = p.ncols_pad / 32;
     dim3 grid(p.nsplit, p.Hkv * colblks, batch);
     hipLaunchKernelGGL((ksa_decode_kernel<T, D>), grid, dim3(kThreads), 0, stream, p);
     if (p.nsplit > 1) {
@@ -304,6 +334,8 @@ int launch(const DecodeParams& p, int batch, hipStream_t stream) {
 }
 
 int pad_cols(int ncols) { return (ncols + 31) / 32 * 32; }
+// column slots of the chunk-boundary form: a block of 32 for the text token, the summary tokens behind it
+int pad_cols_boundary(int Q, int g) { return 32 + pad_cols((Q - 1) * g); }
 
 }  // namespace
 
@@ -332,10 +364,17 @@ int decode_fwd_impl(const void* q, const void* kcache, const void* vcache, void*
                     const int32_t* start, const int32_t* end, int start0, int end0, int batch, int Hq,
                     int Hkv, int Q, int D, int dtype, const int64_t* q_strides,
                     const int64_t* k_strides, const int64_t* v_strides, const int64_t* out_strides,
-                    float scale, int nsplit, void* workspace, size_t workspace_bytes, void* stream) {
+                    float scale, int nsplit, void* workspace, size_t workspace_bytes, void* stream,
+                    bool boundary = false, const int32_t* start2 = nullptr, const int32_t* end2 = nullptr,
+                    int start20 = 0, int end20 = 0) {
     if (!q || !kcache || !vcache || !out || !q_strides || !k_strides || !v_strides || !out_strides)
         return KSA_ERR_NULL;
     if ((start == nullptr) != (end == nullptr)) return KSA_ERR_NULL;
+    if (boundary) {
+        if ((start2 == nullptr) != (end2 == nullptr)) return KSA_ERR_NULL;
+        if (Q < 2 || Hkv <= 0 || Hq % Hkv != 0 || Hq / Hkv > 32) return KSA_ERR_INVALID;
+        if (!start2 && (start20 < 0 || end20 <= start20)) return KSA_ERR_INVALID;
+    }
     if (batch <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || Q <= 0 || nsplit < 1) return KSA_ERR_INVALID;
     if (!start && (start0 < 0 || end0 <= start0)) return KSA_ERR_INVALID;
     if (dtype != KSA_DTYPE_BF16 && dtype != KSA_DTYPE_F16) return KSA_ERR_UNSUPPORTED;
@@ -359,7 +398,9 @@ int decode_fwd_impl(const void* q, const void* kcache, const void* vcache, void*
     p.g = Hq / Hkv;
     p.Q = Q;
     p.ncols = Q * p.g;
-    p.ncols_pad = pad_cols(p.ncols);
+    p.ncols_pad = boundary ? pad_cols_boundary(Q, p.g) : pad_cols(p.ncols);
+    p.split_q = boundary ? 1 : 0;
+    p.start2 = start2, p.end2 = end2, p.start20 = start20, p.end20 = end20;
     p.nsplit = nsplit;
     p.q_bs = q_strides[0], p.q_hs = q_strides[1], p.q_qs = q_strides[2];
     p.k_bs = k_strides[0], p.k_hs = k_strides[1], p.k_rs = k_strides[2];
@@ -367,7 +408,7 @@ int decode_fwd_impl(const void* q, const void* kcache, const void* vcache, void*
     p.o_bs = out_strides[0], p.o_qs = out_strides[1], p.o_hs = out_strides[2];
     p.scale_log2 = scale * 1.4426950408889634f;
     if (nsplit > 1) {
-        const size_t need = ksa_decode_workspace_bytes(batch, Hq, Hkv, Q, D, nsplit);
+        const size_t need = (size_t)batch * Hkv * nsplit * p.ncols_pad * (D + 2) * sizeof(float);
         if (!workspace || workspace_bytes < need) return KSA_ERR_WORKSPACE;
         p.ws_o = (float*)workspace;
         p.ws_ml = p.ws_o + (size_t)batch * Hkv * nsplit * p.ncols_pad * D;
@@ -423,6 +464,28 @@ extern "C" int ksa_decode_fwd(const void* q, const void* kcache, const void* vca
     return decode_fwd_impl(q, kcache, vcache, out, start, end, start0, end0, batch, Hq, Hkv, Q, D, dtype,
                            q_strides, k_strides, v_strides, out_strides, scale, nsplit, workspace,
                            workspace_bytes, stream);
+}
+
+// Chunk-boundary step (HF:831-876): the chunk's last text token and its summary tokens in one launch.
+// Query token 0 attends rows [text_start, text_end) (the slice of get_attention_kv after update_text,
+// HF:844-856), query tokens 1 .. Q - 1 attend [sum_start, sum_end) (the [own summaries | chunk] rows of
+// get_summary_attention_kv, HF:858-870), un-masked both, as the reference's two calls of its decode
+// attention function do; out [batch, Q, Hq, D] is their torch.cat (HF:875).
+extern "C" size_t ksa_decode_boundary_workspace_bytes(int batch, int Hq, int Hkv, int Q, int D, int nsplit) {
+    if (nsplit <= 1 || batch <= 0 || Hkv <= 0 || Hq % Hkv != 0 || Q < 2) return 0;
+    return (size_t)batch * Hkv * nsplit * (size_t)pad_cols_boundary(Q, Hq / Hkv) * (D + 2) * sizeof(float);
+}
+
+extern "C" int ksa_decode_boundary_fwd(const void* q, const void* kcache, const void* vcache, void* out,
+                                       const int32_t* text_start, const int32_t* text_end, int text_start0,
+                                       int text_end0, const int32_t* sum_start, const int32_t* sum_end,
+                                       int sum_start0, int sum_end0, int batch, int Hq, int Hkv, int Q, int D,
+                                       int dtype, const int64_t* q_strides, const int64_t* k_strides,
+                                       const int64_t* v_strides, const int64_t* out_strides, float scale,
+                                       int nsplit, void* workspace, size_t workspace_bytes, void* stream) {
+    return decode_fwd_impl(q, kcache, vcache, out, text_start, text_end, text_start0, text_end0, batch, Hq, Hkv, Q, D,
+                           dtype, q_strides, k_strides, v_strides, out_strides, scale, nsplit, workspace,
+                           workspace_bytes, stream, true, sum_start, sum_end, sum_start0, sum_end0);
 }
 
 extern "C" size_t ksa_decode_noalloc_max_workspace_bytes(void) { return kNoAllocScratchBytes; }

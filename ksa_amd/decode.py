@@ -103,6 +103,52 @@ def ksa_decode(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
     return torch.ops.ksa_amd.decode_fwd(q, kcache, vcache, t_start, t_end, s0, e0, float(scale), int(nsplit))
 
 
+def ksa_decode_boundary(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, text_start, text_end,
+                        sum_start, sum_end, scale: Optional[float] = None,
+                        nsplit: Optional[int] = None) -> torch.Tensor:
+    """The attention of a chunk-boundary step in one launch (modeling_qwen3sa.py:831-876: two calls of
+    the decode attention function and a `torch.cat`): q [b, Hq, 1 + S, D]; query token 0 attends the
+    cache rows [text_start, text_end), the S summary tokens attend [sum_start, sum_end); each bound
+    an int or an int32 GPU tensor [b].  Returns [b, 1 + S, Hq, D]."""
+    assert q.is_cuda and q.dtype in _DTYPES and q.dtype == kcache.dtype == vcache.dtype
+    b, Hq, Q, D = q.shape
+    Hkv, rows = kcache.shape[1], kcache.shape[2]
+    assert Q >= 2 and kcache.shape == vcache.shape and kcache.shape[0] == b and kcache.shape[3] == D and Hq % Hkv == 0
+    assert D in (64, 128, 256), "the boundary form has no padded path: head_dim 64, 128 or 256"
+    if q.stride(-1) != 1:
+        q = q.contiguous()
+    assert kcache.stride(-1) == 1 and vcache.stride(-1) == 1, "cache rows must be contiguous"
+
+    def pair(lo, hi):
+        if torch.is_tensor(lo) or torch.is_tensor(hi):
+            tl = torch.as_tensor(lo, device=q.device).to(torch.int32).expand(b).contiguous()
+            th = torch.as_tensor(hi, device=q.device).to(torch.int32).expand(b).contiguous()
+            return tl, th, 0, 1
+        assert 0 <= int(lo) < int(hi) <= rows, "row range out of bounds"
+        return None, None, int(lo), int(hi)
+    ts, te, ts0, te0 = pair(text_start, text_end)
+    ss, se, ss0, se0 = pair(sum_start, sum_end)
+    if scale is None:
+        scale = float(D) ** -0.5
+    lib = _lib.lib()
+    if nsplit is None:
+        nsplit = lib.ksa_decode_auto_splits(b, Hkv, rows if ts is not None else te0 - ts0)
+    out = torch.empty((b, Q, Hq, D), dtype=q.dtype, device=q.device)
+    ws, ws_bytes = None, 0
+    if nsplit > 1:
+        ws_bytes = lib.ksa_decode_boundary_workspace_bytes(b, Hq, Hkv, Q, D, nsplit)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+    ptr = lambda t: t.data_ptr() if t is not None else None
+    with torch.cuda.device(q.device):
+        rc = lib.ksa_decode_boundary_fwd(
+            q.data_ptr(), kcache.data_ptr(), vcache.data_ptr(), out.data_ptr(), ptr(ts), ptr(te), ts0, te0,
+            ptr(ss), ptr(se), ss0, se0, b, Hq, Hkv, Q, D, _DTYPES[q.dtype], _lib.strides3(q, (0, 1, 2)),
+            _lib.strides3(kcache, (0, 1, 2)), _lib.strides3(vcache, (0, 1, 2)), _lib.strides3(out, (0, 1, 2)),
+            float(scale), int(nsplit), ptr(ws), ws_bytes, _lib.stream_ptr(q.device))
+    _lib.check(rc, "ksa_decode_boundary_fwd")
+    return out
+
+
 def ksa_decode_weights(q: torch.Tensor, kcache: torch.Tensor, start=None, end=None,
                        scale: Optional[float] = None, mask: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The attention probabilities of `ksa_decode`: softmax(q K^T * scale (+ mask)) over the rows

@@ -140,6 +140,8 @@ class HipOps:
         self.add_rmsnorm = elementwise.add_rmsnorm
         self.silu_mul = elementwise.silu_mul
         self._decode = decode.ksa_decode
+        self.decode_boundary = decode.ksa_decode_boundary   # text token + summary tokens of a boundary step, one launch
+        self.move_rows_multi = cache._move_rows_multi        # the step's row moves, one launch for up to eight
         self._linear_rows = gemm.linear_rows
         self._gate_up_silu_rows = gemm.gate_up_silu_rows
         self._argmax_rows = elementwise.argmax_rows
@@ -290,10 +292,11 @@ class KsaQwen3ForCausalLM:
     greedy loop.  All sequences of a batch have the same length."""
 
     # `decode_step_graph` runs this many chunk-boundary steps of a cache eagerly before it records
-    # them: recording the roughly 800 launches of a boundary step costs about as much host time as
-    # three eager boundary steps lose against replayed ones, so a short generation never pays for a
-    # recording it does not use, and a long one pays at most twice the best possible.
-    BOUNDARY_GRAPH_AFTER = 3
+    # them: a replayed boundary step saves about 4 ms against an eager one (7.4 against 11.3 ms at the
+    # 4B shape, batch 8), its recording costs about 24 ms of host time (an eager run outside the
+    # capture first, then the capture), i.e. six boundaries' worth: so a short generation never pays
+    # for a recording it does not use, and a long one pays at most twice the best possible.
+    BOUNDARY_GRAPH_AFTER = 6
 
     def __init__(self, config: KsaQwen3Config, weights: dict, ops=None):
         self.config = config
@@ -318,6 +321,34 @@ class KsaQwen3ForCausalLM:
         if delta is None:
             return self.ops.add_rmsnorm(x, None, w, self.config.rms_norm_eps)
         return self.ops.add_rmsnorm(delta, x, w, self.config.rms_norm_eps)
+
+    def _boundary_attention(self, qh, kh, vh, kc, vc, large, rows):
+        """Attention and cache update of one layer at a chunk-boundary step with the fused operators
+        (`ops.decode_boundary`, `ops.move_rows_multi`): three launches (+ the merge) in place of the
+        reference's sequence (:831-876, :306-398, :476-497: update_text, attention of the text token,
+        summaries into the scratch rows, attention of the summary tokens, flush, append) of twelve.
+        qh [b, Hq, 1 + S, D], kh, vh [b, Hkv, 1 + S, D]; `rows` names the cache rows as
+        `Qwen3RingBufferCache.boundary_slots` does, every value an int or an int32 device tensor [b]:
+        small window: text, start, end, flush_src, flush_dst, flush_rows, append; large window: text,
+        start, end, spare, sum_start, sum_end (= spare - C, spare + S).  Returns [b, 1 + S, Hq, D]."""
+        ops = self.ops
+        C, S = self.config.summary_chunk_size, self.config.summary_token_num
+        kt, vt, ks, vs = kh[:, :, :1], vh[:, :, :1], kh[:, :, 1:], vh[:, :, 1:]
+        if large:
+            # the summary rows sit in spare rows behind the text for the length of the step, so that
+            # [chunk text | own summaries] is one row range
+            sp = rows["spare"]
+            ops.move_rows_multi([(kt, kc, 1, 0, rows["text"]), (vt, vc, 1, 0, rows["text"]),
+                                 (ks, kc, S, 0, sp), (vs, vc, S, 0, sp)])
+            return ops.decode_boundary(qh, kc, vc, rows["start"], rows["end"], rows["sum_start"], rows["sum_end"],
+                                       self.scaling)
+        ops.move_rows_multi([(kt, kc, 1, 0, rows["text"]), (vt, vc, 1, 0, rows["text"]),
+                             (ks, kc, S, 0, 0), (vs, vc, S, 0, 0)])
+        attn = ops.decode_boundary(qh, kc, vc, rows["start"], rows["end"], 0, S + C, self.scaling)
+        ops.move_rows_multi([(kc, kc, rows["flush_rows"], rows["flush_src"], rows["flush_dst"]),
+                             (vc, vc, rows["flush_rows"], rows["flush_src"], rows["flush_dst"]),
+                             (ks, kc, S, 0, rows["append"]), (vs, vc, S, 0, rows["append"])])
+        return attn
 
     def _post_attention(self, lw, attn, x):
         """The second half of a layer at a decode step, from the attention output: (x', delta) with
@@ -481,14 +512,26 @@ class KsaQwen3ForCausalLM:
                 q, k, v = ops.pre_attention(q, k, v, lw["q_norm"], lw["k_norm"], cos, sin, cfg.rms_norm_eps)
                 self._blend_summary(lw, h, sum_rows, cos, sin, q, k, v)
                 qh, kh, vh = q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2)
-                cache.update_text(kh[:, :, :1], vh[:, :, :1], li)
-                a, e = cache.attention_range(li)
-                text_out = ops.decode(qh[:, :, :1], cache.key_cache[li], cache.value_cache[li], a, e,
-                                      self.scaling)
-                k_cs, v_cs = cache.get_summary_attention_kv(li, kh[:, :, 1:], vh[:, :, 1:])
-                sum_out = ops.decode(qh[:, :, 1:], k_cs, v_cs, 0, k_cs.shape[2], self.scaling)
-                cache.update_summary(kh[:, :, 1:], vh[:, :, 1:], li)
-                attn = torch.cat([text_out, sum_out], dim=1)
+                if hasattr(ops, "decode_boundary") and cache.boundary_fits_one_piece(li):
+                    # fused operators: the cache only does the bookkeeping and names the rows
+                    sl = cache.boundary_slots(li, S)
+                    rows = dict(text=sl["text"], start=sl["attend"][0], end=sl["attend"][1])
+                    if cache.is_large_window[li]:
+                        rows.update(spare=sl["spare"], sum_start=sl["spare"] - C, sum_end=sl["spare"] + S)
+                    else:
+                        rows.update(flush_src=sl["flush_src"], flush_dst=sl["flush_dst"],
+                                    flush_rows=sl["flush_rows"], append=sl["append"])
+                    attn = self._boundary_attention(qh, kh, vh, cache.key_cache[li], cache.value_cache[li],
+                                                    cache.is_large_window[li], rows)
+                else:   # the reference's own sequence of cache calls
+                    cache.update_text(kh[:, :, :1], vh[:, :, :1], li)
+                    a, e = cache.attention_range(li)
+                    text_out = ops.decode(qh[:, :, :1], cache.key_cache[li], cache.value_cache[li], a, e,
+                                          self.scaling)
+                    k_cs, v_cs = cache.get_summary_attention_kv(li, kh[:, :, 1:], vh[:, :, 1:])
+                    sum_out = ops.decode(qh[:, :, 1:], k_cs, v_cs, 0, k_cs.shape[2], self.scaling)
+                    cache.update_summary(kh[:, :, 1:], vh[:, :, 1:], li)
+                    attn = torch.cat([text_out, sum_out], dim=1)
             # a text step hands both products straight to the next norm; a boundary step slices them
             if boundary:
                 x, h = self._add_norm(ops.linear(attn.reshape(b, ids.shape[1], -1), lw["o_proj"]), x,
@@ -560,21 +603,29 @@ class KsaQwen3ForCausalLM:
             q, k, v = ops.pre_attention(q, k, v, lw["q_norm"], lw["k_norm"], cos, sin, cfg.rms_norm_eps)
             self._blend_summary(lw, h, sum_rows, cos, sin, q, k, v)
             qh, kh, vh = q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2)
-            mv(kh[:, :, :1], kc, 1, dst_start_seq=bc[kind, 0])
-            mv(vh[:, :, :1], vc, 1, dst_start_seq=bc[kind, 0])
-            text_out = ops.decode(qh[:, :, :1], kc, vc, bc[kind, 1], bc[kind, 2], self.scaling)
-            if kind == 0:
-                mv(kh[:, :, 1:], kc, S, 0, 0)
-                mv(vh[:, :, 1:], vc, S, 0, 0)
-                sum_out = ops.decode(qh[:, :, 1:], kc[:, :, :S + C], vc[:, :, :S + C], 0, S + C, self.scaling)
-                for buf, new in ((kc, kh), (vc, vh)):
-                    mv(buf, buf, C, S, dst_start_seq=bc[0, 3])            # chunk rows -> ring
-                    mv(new[:, :, 1:], buf, S, dst_start_seq=bc[0, 4])     # the chunk's summaries
+            if hasattr(ops, "decode_boundary"):
+                rows = dict(text=bc[kind, 0], start=bc[kind, 1], end=bc[kind, 2])
+                if kind:
+                    rows.update(spare=bc[1, 3], sum_start=bc[1, 4], sum_end=bc[1, 5])
+                else:
+                    rows.update(flush_src=S, flush_rows=C, flush_dst=bc[0, 3], append=bc[0, 4])
+                attn = self._boundary_attention(qh, kh, vh, kc, vc, bool(kind), rows)
             else:
-                mv(kh[:, :, 1:], kc, S, dst_start_seq=bc[1, 3])
-                mv(vh[:, :, 1:], vc, S, dst_start_seq=bc[1, 3])
-                sum_out = ops.decode(qh[:, :, 1:], kc, vc, bc[1, 4], bc[1, 5], self.scaling)
-            attn = torch.cat([text_out, sum_out], dim=1)
+                mv(kh[:, :, :1], kc, 1, dst_start_seq=bc[kind, 0])
+                mv(vh[:, :, :1], vc, 1, dst_start_seq=bc[kind, 0])
+                text_out = ops.decode(qh[:, :, :1], kc, vc, bc[kind, 1], bc[kind, 2], self.scaling)
+                if kind == 0:
+                    mv(kh[:, :, 1:], kc, S, 0, 0)
+                    mv(vh[:, :, 1:], vc, S, 0, 0)
+                    sum_out = ops.decode(qh[:, :, 1:], kc[:, :, :S + C], vc[:, :, :S + C], 0, S + C, self.scaling)
+                    for buf, new in ((kc, kh), (vc, vh)):
+                        mv(buf, buf, C, S, dst_start_seq=bc[0, 3])            # chunk rows -> ring
+                        mv(new[:, :, 1:], buf, S, dst_start_seq=bc[0, 4])     # the chunk's summaries
+                else:
+                    mv(kh[:, :, 1:], kc, S, dst_start_seq=bc[1, 3])
+                    mv(vh[:, :, 1:], vc, S, dst_start_seq=bc[1, 3])
+                    sum_out = ops.decode(qh[:, :, 1:], kc, vc, bc[1, 4], bc[1, 5], self.scaling)
+                attn = torch.cat([text_out, sum_out], dim=1)
             x, h = self._add_norm(ops.linear(attn.reshape(b, 1 + S, -1), lw["o_proj"]), x,
                                   lw["post_attention_layernorm"])
             delta = self._mlp(lw, h)

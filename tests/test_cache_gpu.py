@@ -179,3 +179,32 @@ def test_cache_handoff_at_1024_chunks():
             perr = (pre[0, torch.as_tensor(prow, device=dev).long()].float() - dec[b].float()).abs().max().item()
             print(f"layer {layer} seq {b}: decode vs oracle {err:.2e}, decode vs prefill kernel row {perr:.2e}")
             assert perr <= 2e-2, (layer, b, perr)
+
+
+def test_move_rows_multi_equals_single_moves():
+    """Independent moves in one launch (`ksa_copy_rows_multi`) against the same moves one launch each, in
+    the two groups a chunk-boundary step makes (first the text row and the summary rows into the
+    scratch rows, then the flush of the chunk into the ring and the append of the summaries, for K
+    and for V): strided sources (a transposed projection output), a move inside one buffer, scalar
+    and per-sequence destinations, a zero-row move dropped."""
+    from ksa_amd.cache import _move_rows, _move_rows_multi
+    dev = torch.device("cuda")
+    g = torch.Generator().manual_seed(3)
+    b, H, D, S, C = 3, 2, 128, 8, 128
+    new = torch.randn(b, 1 + S, H, D, generator=g).bfloat16().to(dev).transpose(1, 2)     # [b, H, 1 + S, D], strided
+    bufs = [torch.randn(b, H, 700, D, generator=g).bfloat16().to(dev) for _ in range(2)]
+    ref = [x.clone() for x in bufs]
+    seq = torch.tensor([200, 328, 456], dtype=torch.int32, device=dev)
+    app = torch.tensor([650, 658, 666], dtype=torch.int32, device=dev)
+    for group in (lambda x: [(new[:, :, :1], x, 1, 0, 135), (new[:, :, 1:], x, S, 0, 0), (new, x, 0, 0, 5)],
+                  lambda x: [(x, x, C, S, seq), (new[:, :, 1:], x, S, 0, app)]):
+        _move_rows_multi([m for x in bufs for m in group(x)])
+        for x, r in zip(bufs, ref):
+            for src, dst, n, s0, d0 in group(r):
+                if torch.is_tensor(d0):
+                    _move_rows(src, dst, n, s0, 0, dst_start_seq=d0)
+                else:
+                    _move_rows(src, dst, n, s0, d0)
+        torch.cuda.synchronize()
+        for x, r in zip(bufs, ref):
+            assert torch.equal(x, r)

@@ -253,3 +253,36 @@ def test_eager_attention_forward_signature():
     assert (recon - out.float()).abs().max().item() <= 2e-2
     with pytest.raises(NotImplementedError):
         ksa_amd.eager_attention_forward(M(), q, k, v, torch.zeros(1, device=dev), scaling=1.0)
+
+
+@pytest.mark.parametrize("D,dtype,g", [(128, torch.bfloat16, 4), (128, torch.float16, 1), (64, torch.bfloat16, 2),
+                                       (256, torch.bfloat16, 4)])
+@pytest.mark.parametrize("nsplit", [1, 3, None])
+def test_decode_boundary_equals_two_decodes(D, dtype, g, nsplit):
+    """The chunk-boundary form (text token over its range, the S summary tokens over theirs, one launch)
+    against the two separate launches it stands for - bit for bit at the same split count - and
+    against the oracle; per-sequence text ranges as device tensors with a scalar summary range (the
+    small-window layer of a replayed step), per-sequence ranges for both (large window), and scalars."""
+    import ksa_amd
+    dev = torch.device("cuda")
+    Bz, Hkv, S, C, rows = 3, 2, 8, 128, 1200
+    q, k, v = _mk(Bz, Hkv * g, Hkv, 1 + S, D, rows, seed=17 + D + g, dtype=dtype)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    t0, t1 = np.array([136 - 5, 136 - 128, 136 - 77], np.int32), np.array([1100, 1100, 900], np.int32)
+    cases = [((torch.as_tensor(t0, device=dev), torch.as_tensor(t1, device=dev)), (0, S + C), t0, t1, np.zeros(3, np.int32), np.full(3, S + C, np.int32))]
+    s0, s1 = np.array([700, 650, 820], np.int32), np.array([836, 786, 956], np.int32)
+    cases.append(((torch.as_tensor(np.zeros(3, np.int32), device=dev), torch.as_tensor(s1 - S, device=dev)),
+                  (torch.as_tensor(s0, device=dev), torch.as_tensor(s1, device=dev)), np.zeros(3, np.int32), s1 - S, s0, s1))
+    cases.append(((10, 1111), (0, 136), np.full(3, 10, np.int32), np.full(3, 1111, np.int32), np.zeros(3, np.int32), np.full(3, 136, np.int32)))
+    for (ta, tb), (sa, sb), ta_n, tb_n, sa_n, sb_n in cases:
+        got = ksa_amd.ksa_decode_boundary(qd, kd, vd, ta, tb, sa, sb, nsplit=nsplit)
+        assert got.shape == (Bz, 1 + S, Hkv * g, D)
+        want_t = c_oracle.decode(to_np(q[:, :, :1]), to_np(k), to_np(v), ta_n, tb_n)
+        want_s = c_oracle.decode(to_np(q[:, :, 1:]), to_np(k), to_np(v), sa_n, sb_n)
+        want = np.concatenate([want_t, want_s], axis=1)
+        err = np.abs(to_np(got) - want).max()
+        assert err <= ATOL and err <= RTOL_INF * np.abs(want).max(), err
+        if nsplit is not None:
+            two = torch.cat([ksa_amd.ksa_decode(qd[:, :, :1], kd, vd, ta, tb, nsplit=nsplit),
+                             ksa_amd.ksa_decode(qd[:, :, 1:], kd, vd, sa, sb, nsplit=nsplit)], dim=1)
+            assert torch.equal(got, two)

@@ -4,6 +4,7 @@ bit-identical outputs (same kernels, same arithmetic), on two calls in a row, th
 a smaller problem, so that stale partials of the first call would show.  Called through the C
 ABI (ctypes), outputs and inputs preallocated by the test."""
 import ctypes
+import gc
 
 import numpy as np
 import pytest
@@ -56,13 +57,20 @@ def test_decode_noalloc_matches_workspace_entry_point():
         assert _call(L.ksa_decode_fwd, q, kc, vc, want, start, end, nsplit, ws) == 0
         # nothing may be allocated or freed, neither through torch's allocator nor below it
         # (a hipMalloc inside the library shows in the device's free bytes, not in torch's count)
+        # (garbage of earlier tests collected in the middle of the window would show as a change that
+        # the call did not make: collect it first and keep the collector off for the window)
+        gc.collect()
         torch.cuda.synchronize()
-        before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
-        assert _call(L.ksa_decode_fwd_noalloc, q, kc, vc, got, start, end, nsplit) == 0
-        torch.cuda.synchronize()
-        assert torch.cuda.memory_allocated() == before
-        if seed > 0:   # (the first call on a device may load the library's code object)
-            assert torch.cuda.mem_get_info()[0] == free_before
+        gc.disable()
+        try:
+            before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
+            assert _call(L.ksa_decode_fwd_noalloc, q, kc, vc, got, start, end, nsplit) == 0
+            torch.cuda.synchronize()
+            assert torch.cuda.memory_allocated() == before
+            if seed > 0:   # (the first call on a device may load the library's code object)
+                assert torch.cuda.mem_get_info()[0] == free_before
+        finally:
+            gc.enable()
         assert torch.equal(got.view(torch.int16), want.view(torch.int16)), (seed, b, Hq, Hkv, Q, rows, nsplit)
         ref = c_oracle.decode(q.float().cpu().numpy(), kc.float().cpu().numpy(), vc.float().cpu().numpy(),
                               start.cpu().numpy(), end.cpu().numpy())
