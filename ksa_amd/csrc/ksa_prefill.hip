@@ -264,24 +264,21 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 && D <= 
         return (uint32_t)((kv / mk.S) * Bblk + mk.C + kv % mk.S);
     };
 
-    // tile -> (uniform byte offset, uniform per-load step, per-thread byte offsets)
-    auto tile_src = [&](int n0, uint32_t& ubase, uint32_t& ustep, uint32_t (&voff)[KLD]) {
+    // tile, load i -> (uniform byte offset, uniform per-load step, this thread's byte offset for load i)
+    auto tile_src = [&](int n0, int i, uint32_t& ubase, uint32_t& ustep, uint32_t& voff) {
         const bool in_main = (phys || n0 >= mk.P) && n0 + kTileN <= mk.Sk;
         if (in_main) {
             ubase = (uint32_t)(phys ? n0 : n0 - mk.P) * rb;
             ustep = step_main;
-#pragma unroll
-            for (int i = 0; i < KLD; ++i) voff[i] = thr_main;
+            voff = thr_main;
         } else if (s_fast && n0 + kTileN <= mk.P) {
             ubase = (uint32_t)(n0 / mk.S) * Bblk * rb;
             ustep = step_pre;
-#pragma unroll
-            for (int i = 0; i < KLD; ++i) voff[i] = thr_pre;
+            voff = thr_pre;
         } else {
             ubase = 0;
             ustep = 0;
-#pragma unroll
-            for (int i = 0; i < KLD; ++i) voff[i] = src_row(n0 + ld_row + RSTEP * i) * rb;
+            voff = src_row(n0 + ld_row + RSTEP * i) * rb;
         }
     };
 
@@ -296,16 +293,14 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 && D <= 
     // one 1 KB piece (load i of KLD) of tile n into an LDS tile; `col` = kcol or vcol
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
     auto fill1 = [&](const char* base, uint16_t* tile, uint32_t col, int n, uint32_t word, int i, uint32_t odd_xor) {
-        uint32_t ub, us, vo[KLD];
+        uint32_t ub, us, vo;
         if constexpr (kRegular) {
             const bool in_main = word & 1u;
             ub = word & ~1u;
             us = in_main ? step_main : step_pre;
-            const uint32_t t = in_main ? thr_main : thr_pre;
-#pragma unroll
-            for (int x = 0; x < KLD; ++x) vo[x] = t;
+            vo = in_main ? thr_main : thr_pre;
         } else {
-            tile_src(n * kTileN, ub, us, vo);
+            tile_src(n * kTileN, i, ub, us, vo);
         }
         typedef __attribute__((address_space(3))) char* lptr;
         char* dst = reinterpret_cast<char*>(tile) + (RSTEP * i + wave_u * (64 / CPR)) * ROWB;
@@ -315,7 +310,7 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 && D <= 
         // reads wait for fills it cannot tell apart; which fills must have landed before a
         // barrier is decided by fills_done.
         uint64_t ubase = reinterpret_cast<uint64_t>(base + (ub + us * i));
-        const uint32_t loff = vo[i] + (col ^ ((i & 1) ? odd_xor : 0u));
+        const uint32_t loff = vo + (col ^ ((i & 1) ? odd_xor : 0u));
         uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr)dst;
         if constexpr (D > 128) {
             // (both are the same in every lane; at this size the compiler no longer proves it and

@@ -401,9 +401,20 @@ def test_prefill_other_head_dims(D, dtype):
     (what the reference takes, flash_attn/cute/interface.py:206-209) runs zero-padded at the next
     kernel size with the soft-max scale of the true dimension.  Ragged length, GQA, prefix by
     `summary_pos`, batch 2, lse; against the oracle at the true D."""
+    _other_head_dim_case(D, dtype, 5 * 136 + 77)
+
+
+@pytest.mark.parametrize("D,dtype", [(256, torch.bfloat16), (256, torch.float16), (192, torch.bfloat16)])
+def test_prefill_other_head_dims_regular_shape(D, dtype):
+    """The same at a length whose prefix and key axis are whole tiles (8 chunks: 64 prefix rows, 1152 keys),
+    which takes the kernel variant with regular tile addressing."""
+    _other_head_dim_case(D, dtype, 8 * 136)
+
+
+def _other_head_dim_case(D, dtype, Sq):
     import ksa_amd
     dev = torch.device("cuda")
-    Sq, Hq, Hkv, C, S, W = 5 * 136 + 77, 4, 2, 128, 8, 2
+    Hq, Hkv, C, S, W = 4, 2, 128, 8, 2
     sp = O.summary_positions(Sq, C, S)
     qs, ks, vs = zip(*[make_qkv(Sq, Hq, Hkv, D, seed=70 + b, scaled=False) for b in range(2)])
     q, k, v = (torch.stack(t).to(dtype).to(dev) for t in (qs, ks, vs))
