@@ -28,9 +28,12 @@
 //
 // Masking.  The walk has two phases that are uniform for the workgroup.  Phase A holds
 // the tiles that need no per-element mask: the leading partial tiles below every text
-// row's old-summary bound (there a row is visible as a whole iff it is a text row) and
-// the full tiles.  Phase B holds the remaining partial tiles, masked per element from a
-// 64-bit visibility word per query row.
+// row's old-summary bound (there a row is visible as a whole iff it is a text row), the
+// in-line tiles that lie inside every text row's window and below every row's diagonal and
+// in front of the own chunk of the tile's summary rows (again a row is visible iff it is a
+// text row; the one 8-aligned group of summary columns such a tile may hold is wiped for all
+// rows at once: four registers of the score layout), and the full tiles.  Phase B holds the
+// remaining partial tiles, masked per element from a 64-bit visibility word per query row.
 //
 // Soft-max reference.  The first walk is optimistic: a row's reference exponent comes from
 // the unmasked scores of the first tile and is never moved (no row maximum is computed);
@@ -371,6 +374,7 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 && D <= 
     const int32_t* plist = p.mask_idx + (int64_t)mt * p.idx_stride;
     const int32_t* flist = p.full_idx + (int64_t)mt * p.idx_stride;
     int nquick = 0;
+    int c0 = 0, c1 = 0;  // entries [c0, c1) of the list of partial tiles: the uniform in-line tiles described below
     {
         const int c_first = (mt * kTileM) / Bblk;
         const int w_first = c_first > mk.W ? c_first - mk.W : 0;
@@ -380,23 +384,59 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 && D <= 
         // number of entries of the ascending list below nlim (at most nlim of them): counted by
         // the whole wave, 128 entries per round of independent loads, instead of a binary search
         // whose dependent loads would cost several microseconds at the start of every workgroup
-        const int lim = min(npart, nlim);
-        int cnt = 0;
+        // In-line tiles that every text row of this row tile sees in all their text columns and no summary
+        // row sees at all (entirely inside every text row's [blo, bhi) and in front of the own chunk of the
+        // tile's first summary row): tiles n in [n_c0, n_c1).  They need no per-row mask either - a row is
+        // visible iff it is a text row, and the one group of S = 8 summary columns such a tile may hold is
+        // wiped for all rows at once (see `step`).  With chunks of C + S columns that are multiples of 8
+        // and hold a whole tile, a tile holds at most one such group and the group is 8-aligned in it.
+        int n_c0 = 0, n_c1 = 0;
+#ifndef KSA_PREFILL_NO_UNIFORM_TILES
+        if (mk.S == 8 && mk.C % 8 == 0 && mk.P % 8 == 0 && Bblk >= kTileN + 8) {
+            const int R0 = mt * kTileM, R1 = min(R0 + kTileM, mk.Sq) - 1;
+            const int q_ft = (R0 % Bblk) < mk.C ? R0 : (R0 / Bblk + 1) * Bblk;            // first text row
+            const int q_lt = (R1 % Bblk) < mk.C ? R1 : (R1 / Bblk) * Bblk + mk.C - 1;      // last text row
+            const int q_fs = (R0 % Bblk) >= mk.C ? R0 : (R0 / Bblk) * Bblk + mk.C;          // first summary row
+            if (q_ft <= R1 && q_lt >= q_ft) {
+                const int c_lt = q_lt / Bblk;
+                const int lo = mk.P + (c_lt > mk.W ? c_lt - mk.W : 0) * Bblk;
+                int hi = mk.P + q_ft + 1;
+                if (q_fs <= R1) hi = min(hi, mk.P + (q_fs / Bblk) * Bblk);
+                n_c0 = (lo + kTileN - 1) / kTileN;
+                n_c1 = max(hi / kTileN, n_c0);
+            }
+        }
+#endif
+        // number of entries of the ascending list below nlim (at most nlim of them), below n_c0 and
+        // below n_c1: counted by the whole wave, 128 entries per round of independent loads, instead
+        // of binary searches whose dependent loads would cost several microseconds at the start of
+        // every workgroup
+        const int lim = min(npart, max(nlim, n_c1));
+        int cnt = 0, cnt0 = 0, cnt1 = 0;
         for (int base = 0; base < lim; base += 128) {
             const int i0 = base + lane, i1 = base + 64 + lane;
-            const int e0 = i0 < lim ? plist[i0] : nlim;
-            const int e1 = i1 < lim ? plist[i1] : nlim;
+            const int e0 = i0 < lim ? plist[i0] : 0x7fffffff;
+            const int e1 = i1 < lim ? plist[i1] : 0x7fffffff;
             cnt += __popcll(__ballot(e0 < nlim)) + __popcll(__ballot(e1 < nlim));
+            cnt0 += __popcll(__ballot(e0 < n_c0)) + __popcll(__ballot(e1 < n_c0));
+            cnt1 += __popcll(__ballot(e0 < n_c1)) + __popcll(__ballot(e1 < n_c1));
         }
         nquick = cnt;
+        c0 = max(cnt0, nquick);
+        c1 = max(cnt1, c0);
     }
     const bool last_full_cut = nfull > 0 && (flist[nfull - 1] + 1) * kTileN > mk.Sk;
     const int nfull_a = nfull - (last_full_cut ? 1 : 0);
-    const int n_a = nquick + nfull_a;
+    // Walk order.  Phase A: the leading prefix tiles, the uniform in-line tiles, the full tiles; phase B:
+    // the other partial tiles (those in front of the uniform run, those behind it, a cut full tile).
+    const int ncheap = c1 - c0;
+    const int n_a = nquick + ncheap + nfull_a;
     auto tile_at = [&](int i) {
         if (i < nquick) return plist[i];
-        if (i < n_a) return flist[i - nquick];
-        const int j = i - n_a + nquick;
+        if (i < nquick + ncheap) return plist[c0 + (i - nquick)];
+        if (i < n_a) return flist[i - nquick - ncheap];
+        int j = i - n_a + nquick;            // entries [nquick, c0), then [c1, npart)
+        if (j >= c0) j += ncheap;
         return j < npart ? plist[j] : flist[nfull - 1];
     };
     // The order is kept in registers, 64 entries at a time (lane i holds entry base + i),
@@ -512,6 +552,28 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 && D <= 
         auto vfrag = [&](int j) { return read_v(vsrc, j); };
         __builtin_amdgcn_sched_barrier(0);
 
+        if constexpr (!kGeneral) {
+            if (quick && it >= nquick) {
+                // a uniform in-line tile (see the walk order): if it holds the group of summary columns of a
+                // chunk, those eight keys are hidden from every row - in the score layout they are four
+                // registers of one 32-key block, the same in every lane
+                int rel = mk.C - seq_phase(it, it);
+                rel += rel < 0 ? Bblk : 0;
+                if (rel < kTileN) {
+                    const int gj = rel >> 3;
+#pragma unroll
+                    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                        for (int qd = 0; qd < 4; ++qd)
+                            if (gj == 4 * kb + qd) {
+#pragma unroll
+                                for (int r = 0; r < RB; ++r)
+#pragma unroll
+                                    for (int e = 0; e < 4; ++e) scur[r][kb][4 * qd + e] = -INFINITY;
+                            }
+                }
+            }
+        }
         if constexpr (kGeneral) {  // 64-bit visibility word per row
             const int kv = n0 + lane;
             const bool in = kv < mk.Sk;
@@ -766,11 +828,11 @@ __global__ __launch_bounds__((PrefillShape<RB, HW>::kThreads), (RB == 1 && D <= 
         }
         int it = 0;
         for (; it + 2 <= n_a; it += 2) {
-            step(safe_tag, A{}, Even{}, it, s0, s1, it < nquick);
-            step(safe_tag, A{}, Odd{}, it + 1, s1, s0, it + 1 < nquick);
+            step(safe_tag, A{}, Even{}, it, s0, s1, it < nquick + ncheap);
+            step(safe_tag, A{}, Odd{}, it + 1, s1, s0, it + 1 < nquick + ncheap);
         }
         if (it < n_a) {
-            step(safe_tag, A{}, Even{}, it, s0, s1, it < nquick);
+            step(safe_tag, A{}, Even{}, it, s0, s1, it < nquick + ncheap);
             copy_scores();
             ++it;
         }

@@ -222,6 +222,42 @@ def test_prefill_visibility_probe():
     assert np.abs(got[:, 1] - want).max() <= 4e-3
 
 
+@pytest.mark.parametrize("C", [128, 64, 200, 56])
+@pytest.mark.parametrize("W", [0, 1, 3, 1 << 20])
+@pytest.mark.parametrize("mode", ["prefix", "inline", "skip_old", "physical"])
+def test_prefill_visibility_probe_uniform_tiles(C, W, mode, wave_rows):
+    """The exact probe of `test_prefill_visibility_probe` (Q = K = 0, V = one-hot of position mod D: the
+    output is count-of-class / visible keys, so one wrongly (un)masked key moves a value far beyond the
+    tolerance) over the cases that decide how the in-line tiles are walked: S = 8 with chunk sizes whose
+    period holds a tile (128, 64, 200) and one that does not (56 + 8 < 72: the per-row masks only), windows
+    from none to unbounded (a dense-causal layer: almost every listed tile takes the path that wipes
+    one group of summary columns for all rows), the summary prefix in place / in-line (P = 0) /
+    skipped / carried by k and v, a ragged tail.  Expected values from the dense predicate."""
+    S, D, Hq, Hkv = 8, 128, 2, 1
+    Sq = 11 * (C + S) + C // 2 + 3
+    q = torch.zeros(Sq, Hq, D, dtype=torch.bfloat16)
+    k = torch.zeros(Sq, Hkv, D, dtype=torch.bfloat16)
+    v = torch.zeros(Sq, Hkv, D, dtype=torch.bfloat16)
+    v[torch.arange(Sq), 0, torch.arange(Sq) % D] = 1.0
+    sp = O.summary_positions(Sq, C, S)
+    skip = mode == "skip_old"
+    if mode == "inline":
+        got, _ = _run_prefill(q, k, v, C, S, W, None, False)
+        P = 0
+    elif mode == "physical":
+        spt = torch.as_tensor(sp)
+        got, _ = _run_prefill(q, torch.cat([k[spt], k]), torch.cat([v[spt], v]), C, S, W, None, False)
+        P = int(sp.sum())
+    else:
+        got, _ = _run_prefill(q, k, v, C, S, W, sp, skip)
+        P = int(sp.sum())
+    vis = O.dense_mask_predicate(Sq, C, S, W, P, skip_old=skip)
+    vfull = np.concatenate([to_np(v)[sp], to_np(v)], axis=0)[:, 0, :] if P else to_np(v)[:, 0, :]
+    want = (vis.astype(np.float64) @ vfull) / vis.sum(axis=1, keepdims=True)
+    for h in range(Hq):
+        assert np.abs(got[:, h] - want).max() <= 4e-3, (C, W, mode, h, np.abs(got[:, h] - want).max())
+
+
 def test_prefill_cfg1_sampled_rows(wave_rows):
     """cfg 1 (32k text tokens, 32/8 heads): rows of the first and last two chunks, offsets
     {0, C-1, C, B-1} of 64 random chunks and 1024 random rows against the oracle."""
