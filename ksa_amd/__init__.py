@@ -14,13 +14,12 @@ from .prefill import SUMMARY_ATTN_CACHE, compute_block_sparsity, summary_attn_fu
 from .decode import (decode_attention_forward, eager_attention_forward, ksa_decode, ksa_decode_boundary,  # noqa: E402
                      ksa_decode_weights)
 from .cache import Qwen3RingBufferCache  # noqa: E402
-from .pre import pre_attention  # noqa: E402
-from .elementwise import add_rmsnorm, silu_mul  # noqa: E402
-from .gemm import linear_rows  # noqa: E402
+from . import ops  # noqa: E402  (registers torch.ops.ksa_amd.* for the helper operators)
+from .ops import add_rmsnorm, linear_rows, pre_attention, silu_mul  # noqa: E402
 from .model import KsaQwen3Config, KsaQwen3ForCausalLM, init_weights  # noqa: E402
 
 __all__ = [
     "KsaError", "SUMMARY_ATTN_CACHE", "compute_block_sparsity", "summary_attn_func",
-    "decode_attention_forward", "eager_attention_forward", "ksa_decode", "ksa_decode_boundary", "ksa_decode_weights", "Qwen3RingBufferCache", "pre_attention", "add_rmsnorm", "silu_mul", "linear_rows",
+    "decode_attention_forward", "eager_attention_forward", "ksa_decode", "ksa_decode_boundary", "ksa_decode_weights", "Qwen3RingBufferCache", "pre_attention", "add_rmsnorm", "silu_mul", "linear_rows", "ops",
     "KsaQwen3Config", "KsaQwen3ForCausalLM", "init_weights",
 ]
