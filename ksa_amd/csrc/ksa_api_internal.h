@@ -16,6 +16,9 @@ enum {
 
 enum { KSA_DTYPE_BF16 = 0, KSA_DTYPE_F16 = 1 };
 
+// most rows of x that the few-rows GEMM (ksa_gemm_rows) and the consumers of its K-split partial sums take
+constexpr int kMaxPartialRows = 128;
+
 // size of the fixed device array behind ksa_decode_fwd_noalloc (32 MiB; include/ksa_hip.h states it too)
 #define KSA_DECODE_NOALLOC_SCRATCH_BYTES (32u << 20)
 

@@ -83,10 +83,14 @@ struct KsaCvt<KsaF16> {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-// eight consecutive columns of a row of x = the rounded sum of fp32 slices [ksplit][16][width]
-// (the K-split partial sums of ksa_gemm_rows), added in split order like its own reduction
+// rows of one slice of the K-split partial sums of a product with `rows` rows: whole 16-row blocks
+__host__ __device__ __forceinline__ int ksa_partial_rows(int rows) { return (rows + 15) / 16 * 16; }
+
+// eight consecutive columns of a row of x = the rounded sum of fp32 slices [ksplit][prows][width]
+// (the K-split partial sums of ksa_gemm_rows, prows = ksa_partial_rows(rows of x)), added in split
+// order like its own reduction
 template <typename T>
-__device__ __forceinline__ u32x4 ksa_sum_partials8(const float* part, int ksplit, int width, int row, int col) {
+__device__ __forceinline__ u32x4 ksa_sum_partials8(const float* part, int ksplit, int prows, int width, int row, int col) {
     using C = KsaCvt<T>;
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     for (int sp0 = 0; sp0 < ksplit; sp0 += 8) {  // eight slices requested together
@@ -94,7 +98,7 @@ __device__ __forceinline__ u32x4 ksa_sum_partials8(const float* part, int ksplit
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
             const int sp = min(sp0 + u, ksplit - 1);
-            const float* src = part + ((int64_t)sp * 16 + row) * width + col;
+            const float* src = part + ((int64_t)sp * prows + row) * width + col;
             lo[u] = *reinterpret_cast<const f32x4*>(src);
             hi[u] = *reinterpret_cast<const f32x4*>(src + 4);
         }

@@ -16,7 +16,7 @@ namespace {
 
 struct NormParams {
     const uint16_t* x;
-    const float* part;     // partial-sum variant: x = rounded sum of `ksplit` fp32 slices [ksplit][16][H]
+    const float* part;     // partial-sum variant: x = rounded sum of `ksplit` fp32 slices [ksplit][ksa_partial_rows(rows)][H]
     int ksplit;
     const uint16_t* res;   // may be null
     const uint16_t* w;
@@ -81,7 +81,7 @@ __global__ __launch_bounds__(256) void ksa_add_rmsnorm_kernel(const NormParams p
 }
 
 // The same step for the few rows of a decode step when x is still the K-split partial sums of
-// the GEMM that produced it (fp32 [ksplit][16][H], as ksa_gemm_rows leaves them): one workgroup
+// the GEMM that produced it (fp32 [ksplit][rows in whole 16-row blocks][H], as ksa_gemm_rows leaves them): one workgroup
 // per row, as many threads as the row has 16-byte items (up to 512, then NJ = 2 items per thread),
 // adds the slices in split order, rounds (which is what the GEMM's own reduction does), adds the
 // residual and normalises.  Everything that does not depend on the sums is requested first.
@@ -106,7 +106,7 @@ __global__ __launch_bounds__(512) void ksa_add_rmsnorm_partials_kernel(const Nor
     for (int j = 0; j < NJ; ++j) {
         const int idx = tid + nthr * j;
         if (idx < items) {
-            const u32x4 x = ksa_sum_partials8<T>(p.part, p.ksplit, p.H, row, 8 * idx);
+            const u32x4 x = ksa_sum_partials8<T>(p.part, p.ksplit, ksa_partial_rows(p.rows), p.H, row, 8 * idx);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 r[j][i] = C::down2(C::lo(x[i]) + C::lo(q[j][i]), C::hi(x[i]) + C::hi(q[j][i]));
@@ -192,9 +192,9 @@ __global__ __launch_bounds__(256) void ksa_silu_mul_kernel(const ActParams p) {
     const int idx = blockIdx.y * 256 + threadIdx.x;
     if (idx >= p.I / 8) return;
     u32x4 g, u;
-    if constexpr (kPartials) {  // gate | up still as the partial sums of the fused projection [ksplit][16][2 I]
-        g = ksa_sum_partials8<T>(p.part, p.ksplit, 2 * p.I, (int)row, 8 * idx);
-        u = ksa_sum_partials8<T>(p.part, p.ksplit, 2 * p.I, (int)row, p.I + 8 * idx);
+    if constexpr (kPartials) {  // gate | up still as the partial sums of the fused projection [ksplit][ksa_partial_rows(rows)][2 I]
+        g = ksa_sum_partials8<T>(p.part, p.ksplit, ksa_partial_rows((int)gridDim.x), 2 * p.I, (int)row, 8 * idx);
+        u = ksa_sum_partials8<T>(p.part, p.ksplit, ksa_partial_rows((int)gridDim.x), 2 * p.I, (int)row, p.I + 8 * idx);
     } else {
         g = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.gate + row * p.gs + 8 * idx));
         u = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.up + row * p.us + 8 * idx));
@@ -312,7 +312,7 @@ extern "C" int ksa_add_rmsnorm_partials(const float* partials, int ksplit, const
                                         long long residual_row_stride, long long norm_row_stride,
                                         long long sum_row_stride, int dtype, float eps, void* stream) {
     if (!partials || !residual || !weight || !out_norm || !out_sum) return KSA_ERR_NULL;
-    if (rows <= 0 || rows > 16 || ksplit < 1 || ksplit > 64 || H <= 0 || H % 8 != 0 || !(eps >= 0.f))
+    if (rows <= 0 || rows > kMaxPartialRows || ksplit < 1 || ksplit > 64 || H <= 0 || H % 8 != 0 || !(eps >= 0.f))
         return KSA_ERR_INVALID;
     if (dtype != KSA_DTYPE_BF16 && dtype != KSA_DTYPE_F16) return KSA_ERR_UNSUPPORTED;
     if (!al16(partials) || !al16(residual) || !al16(weight) || !al16(out_norm) || !al16(out_sum)) return KSA_ERR_ALIGN;
@@ -356,7 +356,7 @@ extern "C" int ksa_silu_mul(const void* gate, const void* up, void* out, long lo
 extern "C" int ksa_silu_mul_partials(const float* partials, int ksplit, void* out, int rows, int I,
                                      long long out_row_stride, int dtype, void* stream) {
     if (!partials || !out) return KSA_ERR_NULL;
-    if (rows <= 0 || rows > 16 || ksplit < 1 || ksplit > 64 || I <= 0 || I % 8 != 0) return KSA_ERR_INVALID;
+    if (rows <= 0 || rows > kMaxPartialRows || ksplit < 1 || ksplit > 64 || I <= 0 || I % 8 != 0) return KSA_ERR_INVALID;
     if (dtype != KSA_DTYPE_BF16 && dtype != KSA_DTYPE_F16) return KSA_ERR_UNSUPPORTED;
     if (!al16(partials) || !al16(out) || out_row_stride % 8) return KSA_ERR_ALIGN;
     const int yblocks = (I / 8 + 255) / 256;

@@ -8,8 +8,12 @@
 // of W, quarter of the 32-wide K step): 16 contiguous bytes per lane, 64 contiguous bytes per
 // row and instruction), the rows of x, staged in LDS, are the B operand.  With more than one K
 // split per column tile the fp32 partial sums go to a workspace and a second kernel adds and
-// rounds them.
+// rounds them.  Up to 16 rows of x are one B operand; 17 to 128 rows (a decode step of a larger batch,
+// the 9 tokens per sequence of a chunk-boundary step) take the `wide` kernel below, which feeds every
+// weight fragment to one MFMA per 16-row block of x.
 #include <hip/hip_runtime.h>
+
+#include <type_traits>
 
 #include "ksa_api_internal.h"
 #include "ksa_cvt.h"
@@ -21,7 +25,7 @@ struct GemmParams {
     const uint16_t* x;   // [M, K], row stride xs
     const uint16_t* w;   // [N, K], row stride ws
     uint16_t* out;       // [M, N], row stride os
-    float* part;         // [ksplit, 16, N] when ksplit > 1
+    float* part;         // [ksplit, ksa_partial_rows(M), N] when ksplit > 1
     int64_t xs, ws, os;
     int M, N, K, ksplit;
 };
@@ -96,8 +100,247 @@ __global__ __launch_bounds__(256) void ksa_gemm_rows_reduce_kernel(const GemmPar
     if (e >= (int64_t)p.M * p.N) return;
     const int m = (int)(e / p.N), n = (int)(e % p.N);
     float v = 0.f;
-    for (int sp = 0; sp < p.ksplit; ++sp) v += p.part[((int64_t)sp * 16 + m) * p.N + n];
+    const int prows = ksa_partial_rows(p.M);
+    for (int sp = 0; sp < p.ksplit; ++sp) v += p.part[((int64_t)sp * prows + m) * p.N + n];
     p.out[(int64_t)m * p.os + n] = C::down(v);
+}
+
+
+// ---- 17 to 128 rows of x ----
+// grid: (column tiles, K splits); block: eight waves, each 16 columns over the K slice of the
+// workgroup, which it walks in chunks of 512 elements.  Per chunk the workgroup stages the rows of x in
+// LDS once (one buffer: 1040 bytes per row, whole 16-row blocks, up to 130 KB) and every wave multiplies its 16 weight fragments
+// with each of the MB 16-row blocks of x.  The stream from HBM does not stop at the two barriers between
+// chunks: a weight fragment's register is refilled with the next chunk's fragment right behind its last
+// MFMA, and the next chunk of x waits in registers, requested in front of those (so that the wait for it
+// does not include them).
+// kPair (the MLP's first half, out = SiLU(x Wg^T) * (x Wu^T) with w = [gate rows; up rows]): waves
+// 0..3 take gate columns, waves 4..7 the same columns of up; they meet in LDS behind the walk and the
+// up waves write the activation.  K is not split in this form.
+struct WideParams {
+    const uint16_t* x;
+    const uint16_t* w;
+    uint16_t* out;
+    float* part;  // [ksplit, ksa_partial_rows(M), N] when ksplit > 1
+    int64_t xs, ws, os;
+    int M, N, K, ksplit, chunks_per_split;
+};
+constexpr int kWideWaves = 8;
+
+template <typename T, int MB, bool kPair>
+__global__ __launch_bounds__(64 * kWideWaves) void ksa_gemm_rows_wide_kernel(const WideParams p) {
+    using C = KsaCvt<T>;
+    extern __shared__ __attribute__((aligned(16))) unsigned char wide_lds[];
+    constexpr int nw = kWideWaves;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int r = lane & 15;   // row of W inside the wave's tile (A operand) / row of x inside a block (B operand)
+    const int kq = lane >> 4;  // which 8 of the 32 K elements of a step
+    int n0;                    // first output column of this wave (kPair: of the gate / up half)
+    int64_t wrow;              // this lane's row of w
+    if constexpr (kPair) {
+        const int half = wave / (nw / 2);
+        n0 = (blockIdx.x * (nw / 2) + wave % (nw / 2)) * 16;
+        wrow = (int64_t)half * p.N + min(n0 + r, p.N - 1);
+    } else {
+        n0 = (blockIdx.x * nw + wave) * 16;
+        wrow = min(n0 + r, p.N - 1);
+    }
+    const int steps = p.K / 32;
+    const int chunks = (steps + kChunkSteps - 1) / kChunkSteps;
+    const int c_begin = blockIdx.y * p.chunks_per_split;
+    const int c_end = min(chunks, c_begin + p.chunks_per_split);
+    const uint16_t* wp = p.w + wrow * p.ws + 8 * kq;
+
+    f32x4 acc[MB];
+#pragma unroll
+    for (int b = 0; b < MB; ++b) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+    // rows of x beyond M repeat the last one: their columns of the product are never stored
+    int xoff[MB];
+#pragma unroll
+    for (int b = 0; b < MB; ++b) xoff[b] = min(16 * b + r, p.M - 1) * kRowB + 16 * kq;
+
+    // staging of a chunk of x: thread = (row tr of a pass of eight rows, 16-byte piece tj of the row's chunk).
+    // No predicates: rows past M repeat the last row and pieces past a short last chunk its last piece
+    // (LDS holds whole 16-row blocks; what lands there is never used).
+    constexpr int XT = 2 * MB;
+    const int tr = threadIdx.x >> 6, tj = threadIdx.x & 63;
+    unsigned char* xdst = wide_lds + tr * kRowB + 16 * tj;
+    int64_t xrow_off[XT];
+#pragma unroll
+    for (int i = 0; i < XT; ++i) xrow_off[i] = (int64_t)min(tr + nw * i, p.M - 1) * p.xs;
+    u32x4 xt[XT];
+    auto x_request = [&](int c) {
+        const int nst = min(kChunkSteps, steps - c * kChunkSteps);
+        const uint16_t* src = p.x + (int64_t)kChunkK * c + 8 * min(tj, 4 * nst - 1);
+#pragma unroll
+        for (int i = 0; i < XT; ++i) xt[i] = *reinterpret_cast<const u32x4*>(src + xrow_off[i]);
+    };
+    // (a short last chunk is filled up with zeros: its missing steps then add nothing, whatever weights
+    // the clamped requests fetch for them)
+    auto x_store = [&](int c) {
+        const bool live = tj < 4 * min(kChunkSteps, steps - c * kChunkSteps);
+#pragma unroll
+        for (int i = 0; i < XT; ++i) {
+            u32x4 v = xt[i];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = live ? v[e] : 0u;
+            *reinterpret_cast<u32x4*>(xdst + nw * i * kRowB) = v;
+        }
+    };
+    u32x4 a[kChunkSteps];
+    auto w_request = [&](int c, int u) {
+        a[u] = *reinterpret_cast<const u32x4*>(wp + 32 * min(c * kChunkSteps + u, steps - 1));
+    };
+    // the products of one chunk; kMore: there is a next chunk, whose x and weights are requested on the way
+    // (two copies of the loop body rather than a condition inside it: with branches between the MFMAs the
+    // compiler waits for every outstanding load in front of each of them)
+    auto chunk = [&](auto more_tag, int cn) __attribute__((always_inline)) {  // cn: the next chunk (kMore)
+        constexpr bool kMore = decltype(more_tag)::value;
+        if constexpr (kMore) x_request(cn);
+        // the rows of x of step u + 1 are read from LDS while the MFMAs of step u run; the fences keep
+        // the compiler from reading many steps ahead (which costs it more registers than there are)
+        u32x4 bf[2][MB];
+#pragma unroll
+        for (int b = 0; b < MB; ++b) bf[0][b] = *reinterpret_cast<const u32x4*>(wide_lds + xoff[b]);
+#pragma unroll
+        for (int u = 0; u < kChunkSteps; ++u) {
+            if (u + 1 < kChunkSteps) {
+#pragma unroll
+                for (int b = 0; b < MB; ++b)
+                    bf[(u + 1) & 1][b] = *reinterpret_cast<const u32x4*>(wide_lds + xoff[b] + 64 * (u + 1));
+            }
+#pragma unroll
+            for (int b = 0; b < MB; ++b) acc[b] = mfma16<T>(a[u], bf[u & 1][b], acc[b]);
+            if constexpr (kMore) w_request(cn, u);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    if (c_begin < c_end) {  // (uniform; an empty slice does not exist in a grid made by wide_plan)
+        // The workgroups of a launch walk their chunks in rotated orders: rows of w are K elements apart,
+        // and with every workgroup at the same offset inside its rows at the same time the requests of the
+        // whole grid meet in a few memory channels.
+        const int nch = c_end - c_begin;
+        int c = c_begin + (int)(blockIdx.x % (unsigned)nch);
+        auto next = [&](int cc) { return cc + 1 < c_end ? cc + 1 : c_begin; };
+        x_request(c);
+#pragma unroll
+        for (int u = 0; u < kChunkSteps; ++u) w_request(c, u);
+        x_store(c);
+        __syncthreads();
+        for (int k = 0; k + 1 < nch; ++k) {
+            const int cn = next(c);
+            chunk(std::true_type{}, cn);
+            __syncthreads();  // every wave is done with this chunk of x
+            x_store(cn);
+            __syncthreads();
+            c = cn;
+        }
+        chunk(std::false_type{}, c);
+    }
+    // C layout of a 16x16 tile: lane holds row (of x) lane % 16 of the block, columns n0 + 4 * (lane / 16) + i
+    const int n = n0 + 4 * kq;
+    if constexpr (kPair) {
+        __syncthreads();  // x is no longer read: its place takes the gate halves
+        f32x4* ex = reinterpret_cast<f32x4*>(wide_lds);
+        constexpr int hw = nw / 2;
+        if (wave < hw) {
+#pragma unroll
+            for (int b = 0; b < MB; ++b) ex[(wave * MB + b) * 64 + lane] = acc[b];
+        }
+        __syncthreads();
+        if (wave >= hw) {
+#pragma unroll
+            for (int b = 0; b < MB; ++b) {
+                const int m = 16 * b + r;
+                if (m < p.M && n < p.N) {
+                    const f32x4 gv = ex[((wave - hw) * MB + b) * 64 + lane];
+                    uint16_t o[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const float g = C::up(C::down(gv[i])), u = C::up(C::down(acc[b][i]));
+                        const float act = C::up(C::down(g / (1.f + expf(-g))));
+                        o[i] = C::down(act * u);
+                    }
+                    uint16_t* dst = p.out + (int64_t)m * p.os + n;
+                    if (n + 3 < p.N && (p.os % 4) == 0) {
+                        u32x2 v2;
+                        v2[0] = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
+                        v2[1] = (uint32_t)o[2] | ((uint32_t)o[3] << 16);
+                        *reinterpret_cast<u32x2*>(dst) = v2;
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)
+                            if (n + i < p.N) dst[i] = o[i];
+                    }
+                }
+            }
+        }
+    } else {
+        const int prows = ksa_partial_rows(p.M);
+#pragma unroll
+        for (int b = 0; b < MB; ++b) {
+            const int m = 16 * b + r;
+            if (m < p.M && n < p.N) {
+                if (p.ksplit == 1) {
+                    uint16_t* dst = p.out + (int64_t)m * p.os + n;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        if (n + i < p.N) dst[i] = C::down(acc[b][i]);
+                } else {
+                    float* dst = p.part + ((int64_t)blockIdx.y * prows + m) * p.N + n;
+                    if (n + 3 < p.N && (p.N % 4) == 0) {
+                        *reinterpret_cast<f32x4*>(dst) = acc[b];
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)
+                            if (n + i < p.N) dst[i] = acc[b][i];
+                    }
+                }
+            }
+        }
+    }
+}
+
+// K splits and chunks per split of the wide kernel for a wanted number of splits (slices are whole
+// chunks, none empty)
+struct WidePlan {
+    int ksplit, chunks_per_split;
+};
+static WidePlan wide_plan(int K, int want_splits) {
+    const int chunks = (K / 32 + kChunkSteps - 1) / kChunkSteps;
+    WidePlan pl;
+    int sp = want_splits < 1 ? 1 : want_splits;
+    if (sp > chunks) sp = chunks;
+    pl.chunks_per_split = (chunks + sp - 1) / sp;
+    pl.ksplit = (chunks + pl.chunks_per_split - 1) / pl.chunks_per_split;
+    return pl;
+}
+
+template <typename T, bool kPair>
+int launch_wide(const WideParams& p, hipStream_t st) {
+    const int mb = (p.M + 15) / 16;
+    constexpr int cols = kPair ? 16 * (kWideWaves / 2) : 16 * kWideWaves;
+    const dim3 grid((p.N + cols - 1) / cols, p.ksplit), block(64 * kWideWaves);
+    size_t lds = (size_t)mb * 16 * kRowB;
+    if (kPair && lds < (size_t)(kWideWaves / 2) * mb * 64 * sizeof(f32x4)) lds = (size_t)(kWideWaves / 2) * mb * 64 * sizeof(f32x4);
+    if (lds > 160 * 1024) return KSA_ERR_UNSUPPORTED;
+    auto go = [&](auto kern) {
+        if (lds > 64 * 1024 &&
+            hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)lds) != hipSuccess)
+            return (int)KSA_ERR_LAUNCH;
+        hipLaunchKernelGGL(kern, grid, block, lds, st, p);
+        return ksa_check_launch();
+    };
+    switch (mb) {
+        case 2: return go(ksa_gemm_rows_wide_kernel<T, 2, kPair>);
+        case 3: return go(ksa_gemm_rows_wide_kernel<T, 3, kPair>);
+        case 4: return go(ksa_gemm_rows_wide_kernel<T, 4, kPair>);
+        case 5: return go(ksa_gemm_rows_wide_kernel<T, 5, kPair>);
+        case 6: return go(ksa_gemm_rows_wide_kernel<T, 6, kPair>);
+        default: return go(ksa_gemm_rows_wide_kernel<T, 8, kPair>);
+    }
 }
 
 template <typename T>
@@ -228,15 +471,59 @@ extern "C" size_t ksa_gemm_rows_workspace_bytes(int N, int ksplit) {
     return ksplit > 1 ? (size_t)ksplit * 16 * (size_t)N * sizeof(float) : 0;
 }
 
+// The same two questions for a product of M rows (M <= 16: the answers above).  For more rows a slice
+// of the partial sums has ksa_partial_rows(M) rows, and K is split as far as the grid (tiles of 128
+// columns x splits) stays within about one workgroup per CU - one resident workgroup is all a CU holds
+// of this kernel, and a second round costs more than longer slices do (measured at 72 rows on the
+// projections of the 4B shape: 6144 x 2560 best at 5 splits, 2560 x 4096 at 8, 2560 x 9728 at 10,
+// 19456 x 2560 at 2).
+extern "C" int ksa_gemm_rows_splits(int M, int N, int K) {
+    if (M <= 16) return ksa_gemm_rows_auto_splits(N, K);
+    if (N <= 0 || K <= 0) return 1;
+    const int tiles = (N + 127) / 128;
+    const int want = (ksa_cu_count_or(256) * 5 / 4) / tiles;
+    return wide_plan(K, want).ksplit;
+}
+
+extern "C" size_t ksa_gemm_rows_partials_bytes(int M, int N, int ksplit) {
+    return ksplit > 1 ? (size_t)ksplit * (size_t)ksa_partial_rows(M) * (size_t)N * sizeof(float) : 0;
+}
+
 extern "C" int ksa_gemm_rows(const void* x, const void* w, void* out, int M, int N, int K, long long x_row_stride,
                              long long w_row_stride, long long out_row_stride, int dtype, int ksplit,
                              void* workspace, size_t workspace_bytes, void* stream) {
     if (!x || !w) return KSA_ERR_NULL;
     if (!out && ksplit <= 1) return KSA_ERR_NULL;  // out may be null only to leave the partial sums to the caller
-    if (M <= 0 || M > 16 || N <= 0 || K <= 0 || K % 32 != 0 || ksplit < 1 || ksplit > 64) return KSA_ERR_INVALID;
+    if (M <= 0 || M > kMaxPartialRows || N <= 0 || K <= 0 || K % 32 != 0 || ksplit < 1 || ksplit > 64) return KSA_ERR_INVALID;
     if (dtype != KSA_DTYPE_BF16 && dtype != KSA_DTYPE_F16) return KSA_ERR_UNSUPPORTED;
     if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w)) & 15) return KSA_ERR_ALIGN;
     if (x_row_stride % 8 || w_row_stride % 8) return KSA_ERR_ALIGN;
+    if (M > 16) {
+        const WidePlan pl = wide_plan(K, ksplit);
+        if (pl.ksplit != ksplit) return KSA_ERR_INVALID;  // not a split count of ksa_gemm_rows_splits: an empty slice
+        WideParams wp{};
+        wp.x = (const uint16_t*)x, wp.w = (const uint16_t*)w, wp.out = (uint16_t*)out;
+        wp.xs = x_row_stride, wp.ws = w_row_stride, wp.os = out_row_stride;
+        wp.M = M, wp.N = N, wp.K = K, wp.ksplit = ksplit, wp.chunks_per_split = pl.chunks_per_split;
+        if (ksplit > 1) {
+            if (!workspace || workspace_bytes < ksa_gemm_rows_partials_bytes(M, N, ksplit)) return KSA_ERR_WORKSPACE;
+            wp.part = (float*)workspace;
+        }
+        const int rc = dtype == KSA_DTYPE_BF16 ? launch_wide<KsaBf16, false>(wp, (hipStream_t)stream)
+                                               : launch_wide<KsaF16, false>(wp, (hipStream_t)stream);
+        if (rc != KSA_OK || ksplit == 1 || !out) return rc;
+        GemmParams rp{};
+        rp.out = (uint16_t*)out, rp.part = wp.part, rp.os = out_row_stride;
+        rp.M = M, rp.N = N, rp.K = K, rp.ksplit = ksplit;
+        const int64_t n = (int64_t)M * N;
+        if (dtype == KSA_DTYPE_BF16)
+            hipLaunchKernelGGL(ksa_gemm_rows_reduce_kernel<KsaBf16>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                               (hipStream_t)stream, rp);
+        else
+            hipLaunchKernelGGL(ksa_gemm_rows_reduce_kernel<KsaF16>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                               (hipStream_t)stream, rp);
+        return ksa_check_launch();
+    }
     GemmParams p{};
     p.x = (const uint16_t*)x;
     p.w = (const uint16_t*)w;
@@ -255,10 +542,19 @@ extern "C" int ksa_gemm_rows_gate_up_silu(const void* x, const void* w, void* ou
                                           long long x_row_stride, long long w_row_stride,
                                           long long out_row_stride, int dtype, void* stream) {
     if (!x || !w || !out) return KSA_ERR_NULL;
-    if (M <= 0 || M > 16 || I <= 0 || K <= 0 || K % 32 != 0) return KSA_ERR_INVALID;
+    if (M <= 0 || M > kMaxPartialRows || I <= 0 || K <= 0 || K % 32 != 0) return KSA_ERR_INVALID;
     if (dtype != KSA_DTYPE_BF16 && dtype != KSA_DTYPE_F16) return KSA_ERR_UNSUPPORTED;
     if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w)) & 15) return KSA_ERR_ALIGN;
     if (x_row_stride % 8 || w_row_stride % 8) return KSA_ERR_ALIGN;
+    if (M > 16) {  // chunks of x through LDS, gate and up waves of a workgroup meet behind the walk
+        WideParams wp{};
+        wp.x = (const uint16_t*)x, wp.w = (const uint16_t*)w, wp.out = (uint16_t*)out;
+        wp.xs = x_row_stride, wp.ws = w_row_stride, wp.os = out_row_stride;
+        wp.M = M, wp.N = I, wp.K = K, wp.ksplit = 1;
+        wp.chunks_per_split = (K / 32 + kChunkSteps - 1) / kChunkSteps;
+        return dtype == KSA_DTYPE_BF16 ? launch_wide<KsaBf16, true>(wp, (hipStream_t)stream)
+                                       : launch_wide<KsaF16, true>(wp, (hipStream_t)stream);
+    }
     GateUpParams p{};
     p.x = (const uint16_t*)x;
     p.w = (const uint16_t*)w;

@@ -29,7 +29,7 @@ struct PreParams {
     uint16_t* dst[3];         // q, k, v outputs
     const uint16_t* w[2];     // q_norm, k_norm weights [D]
     const int32_t* kv_row;    // [batch] or null: row added to the k / v destination of a sequence
-    const float* part;        // if set: q | k | v rows as K-split partial sums [ksplit][16][(Hq + 2 Hkv) D], src unused
+    const float* part;        // if set: q | k | v rows as K-split partial sums [ksplit][ksa_partial_rows(batch S)][(Hq + 2 Hkv) D], src unused
     int ksplit;
     const uint16_t* cos;      // [batch or 1, S, D]
     const uint16_t* sin;
@@ -170,7 +170,7 @@ __global__ __launch_bounds__(256) void ksa_pre_attention_kernel(const PreParams 
     // the K-split partial sums of the projection, added and rounded as its own reduction would
     auto fetch = [&](const Group& g) {
         if constexpr (kPartials)
-            return ksa_sum_partials8<T>(p.part, p.ksplit, (p.Hq + 2 * p.Hkv) * D, g.tok, g.col0 + sub * D + 8 * t);
+            return ksa_sum_partials8<T>(p.part, p.ksplit, ksa_partial_rows(ntok), (p.Hq + 2 * p.Hkv) * D, g.tok, g.col0 + sub * D + 8 * t);
         return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(g.sbase + pick(g.which, lsrc)));
     };
 
@@ -264,7 +264,7 @@ int launch_pre(PreParams p, hipStream_t stream) {
     const int64_t blocks = ((int64_t)p.batch * p.S + span - 1) / span;
     // a decode step (one pass of one token per workgroup): one workgroup per four row groups of a
     // token instead of one per token - the groups of a wave are a chain of dependent loads
-    const int parts = (p.passes_per_wg == 1 && p.tok_per_pass == 1 && blocks <= 64) ? G / 4 : 1;
+    const int parts = (p.passes_per_wg == 1 && p.tok_per_pass == 1 && blocks <= kMaxPartialRows) ? G / 4 : 1;
     const dim3 grid((unsigned)blocks, (unsigned)parts);
     if (p.part)
         hipLaunchKernelGGL((ksa_pre_attention_kernel<T, D, true>), grid, dim3(256), 0, stream, p);
@@ -339,7 +339,7 @@ extern "C" int ksa_pre_attention_partials(const float* partials, int ksplit, con
                                           const int32_t* kv_out_row_seq, float eps, void* stream) {
     if (!partials || !q_weight || !k_weight || !cos || !sin || !q_out || !k_out || !v_out) return KSA_ERR_NULL;
     if (!q_out_strides || !k_out_strides || !v_out_strides || !cos_strides) return KSA_ERR_NULL;
-    if (batch <= 0 || S <= 0 || (int64_t)batch * S > 16 || Hq <= 0 || Hkv <= 0 || ksplit < 1 || ksplit > 64 ||
+    if (batch <= 0 || S <= 0 || (int64_t)batch * S > kMaxPartialRows || Hq <= 0 || Hkv <= 0 || ksplit < 1 || ksplit > 64 ||
         !(eps >= 0.f))
         return KSA_ERR_INVALID;
     for (const int64_t* s3 : {q_out_strides, k_out_strides, v_out_strides})

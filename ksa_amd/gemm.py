@@ -2,8 +2,9 @@
 
 Stands in for `torch.nn.functional.linear` (bias-free, as the reference's projections are:
 examples/pretrain/hf_template/modeling_qwen3sa.py:628-641, :507-514, :1338) when x has at most
-16 rows; anything larger should stay a library GEMM.  fp32 accumulation, one rounding at the
-end.  No fallback: without libksa_hip.so it raises.
+128 rows (up to 16: one MFMA operand; 17 to 128, a larger batch or the 9 tokens per sequence of a
+chunk-boundary step: the kernel's wide form); anything larger should stay a library GEMM.  fp32
+accumulation, one rounding at the end.  No fallback: without libksa_hip.so it raises.
 """
 from __future__ import annotations
 
@@ -12,12 +13,13 @@ import torch
 from . import _lib
 
 _DT = {torch.bfloat16: 0, torch.float16: 1}
-MAX_ROWS = 16
+MAX_ROWS = 128       # rows of x the GEMM kernels take
+MLP_MAX_ROWS = 16    # rows the one-launch MLP takes (x whole in LDS)
 
 
 class SplitKPartials:
     """Output of `linear_rows(..., defer=True)` when K was split over workgroups: the fp32 partial
-    sums [ksplit, 16, N] as the kernel left them, for a consumer that adds them itself
+    sums [ksplit, rows rounded up to whole 16-row blocks, N] as the kernel left them, for a consumer that adds them itself
     (`ksa_amd.add_rmsnorm`).  `shape` / `dtype` are those of the tensor it stands for."""
 
     def __init__(self, workspace: torch.Tensor, ksplit: int, rows: int, shape, dtype):
@@ -29,7 +31,7 @@ class SplitKPartials:
 
 
 def linear_rows(x: torch.Tensor, weight: torch.Tensor, defer: bool = False):
-    """x [..., K] with at most 16 rows in all, weight [N, K] -> [..., N].  With `defer`, a product
+    """x [..., K] with at most 128 rows in all, weight [N, K] -> [..., N].  With `defer`, a product
     whose K is split over workgroups comes back as `SplitKPartials` (no reduction launch)."""
     assert x.is_cuda and x.dtype in _DT and weight.dtype == x.dtype, "bf16/fp16 GPU tensors"
     K = x.shape[-1]
@@ -39,15 +41,16 @@ def linear_rows(x: torch.Tensor, weight: torch.Tensor, defer: bool = False):
     if x2.stride(1) != 1:
         x2 = x2.contiguous()
     M = x2.shape[0]
-    assert 1 <= M <= MAX_ROWS, "linear_rows is for at most 16 rows"
+    assert 1 <= M <= MAX_ROWS, "linear_rows is for at most 128 rows"
     L = _lib.lib()
-    ks = L.ksa_gemm_rows_auto_splits(N, K)
+    with torch.cuda.device(x.device):
+        ks = L.ksa_gemm_rows_splits(M, N, K)
     defer = defer and ks > 1
     out = None if defer else torch.empty(M, N, dtype=x.dtype, device=x.device)
     ws = None
     ws_bytes = 0
     if ks > 1:
-        ws_bytes = L.ksa_gemm_rows_workspace_bytes(N, ks)
+        ws_bytes = L.ksa_gemm_rows_partials_bytes(M, N, ks)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
     with torch.cuda.device(x.device):
         rc = L.ksa_gemm_rows(x2.data_ptr(), weight.data_ptr(), None if defer else out.data_ptr(), M, N, K,
@@ -60,7 +63,7 @@ def linear_rows(x: torch.Tensor, weight: torch.Tensor, defer: bool = False):
 
 
 def gate_up_silu_rows(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
-    """x [..., K] with at most 16 rows in all, weight [2 I, K] (gate rows, then up rows) ->
+    """x [..., K] with at most 128 rows in all, weight [2 I, K] (gate rows, then up rows) ->
     SiLU(x W_gate^T) * (x W_up^T) [..., I] in one launch (`ksa_gemm_rows_gate_up_silu`): the MLP's
     `act_fn(gate_proj(x)) * up_proj(x)` (modeling_qwen3sa.py:507-514) at a decode step."""
     assert x.is_cuda and x.dtype in _DT and weight.dtype == x.dtype, "bf16/fp16 GPU tensors"
@@ -71,7 +74,7 @@ def gate_up_silu_rows(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     if x2.stride(1) != 1:
         x2 = x2.contiguous()
     M = x2.shape[0]
-    assert 1 <= M <= MAX_ROWS, "gate_up_silu_rows is for at most 16 rows"
+    assert 1 <= M <= MAX_ROWS, "gate_up_silu_rows is for at most 128 rows"
     out = torch.empty(M, I, dtype=x.dtype, device=x.device)
     with torch.cuda.device(x.device):
         rc = _lib.lib().ksa_gemm_rows_gate_up_silu(x2.data_ptr(), weight.data_ptr(), out.data_ptr(), M, I, K,
@@ -111,7 +114,7 @@ class MlpRowsWorkspace:
 
 
 def mlp_rows_supported(M: int, H: int, I: int) -> bool:
-    return (1 <= M <= MAX_ROWS and H % 128 == 0 and I % 32 == 0 and I <= 26624
+    return (1 <= M <= MLP_MAX_ROWS and H % 128 == 0 and I % 32 == 0 and I <= 26624
             and M * (H + 8) * 2 <= 160 * 1024)
 
 

@@ -211,7 +211,7 @@ class HipOps:
         a decode step, the library GEMM and the activation kernel otherwise."""
         rows = x.numel() // x.shape[-1]
         k = x.shape[-1]
-        if rows <= self._max_rows and k % 32 == 0 and rows * (k + 8) * 2 <= 160 * 1024:
+        if rows <= self._max_rows and k % 32 == 0 and (rows > 16 or rows * (k + 8) * 2 <= 160 * 1024):
             return self._gate_up_silu_rows(x, weight)
         if rows <= self._max_rows:
             return self.silu_mul(self._linear_rows(x, weight, defer=True))
@@ -321,6 +321,30 @@ class KsaQwen3ForCausalLM:
         if delta is None:
             return self.ops.add_rmsnorm(x, None, w, self.config.rms_norm_eps)
         return self.ops.add_rmsnorm(delta, x, w, self.config.rms_norm_eps)
+
+    def _boundary_qkv(self, lw, h, sum_rows, cos, sin):
+        """q, k, v [b, 1 + S, H, D] (normalised, rotated) of a chunk-boundary step's rows.  With one
+        set of projection weights the product may stay the K-split partial sums of the few-rows GEMM,
+        which the pre-attention kernel adds itself (one launch less)."""
+        cfg, ops = self.config, self.ops
+        qkv = None
+        if not cfg.summary_independent_parameters and hasattr(ops, "pre_attention_partials"):
+            qkv = ops.linear(h, lw["qkv_proj"], defer=True)
+        if qkv is not None and not torch.is_tensor(qkv):
+            return ops.pre_attention_partials(qkv, cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim,
+                                              lw["q_norm"], lw["k_norm"], cos, sin, cfg.rms_norm_eps)
+        q, k, v = self._split_qkv(qkv) if qkv is not None else self._qkv(lw, h, sum_rows)
+        q, k, v = ops.pre_attention(q, k, v, lw["q_norm"], lw["k_norm"], cos, sin, cfg.rms_norm_eps)
+        self._blend_summary(lw, h, sum_rows, cos, sin, q, k, v)
+        return q, k, v
+
+    def _boundary_logits(self, x, delta):
+        """Logits of the text rows (row 0 of every sequence) behind the last layer of a boundary step."""
+        if torch.is_tensor(delta):
+            return self._logits(x[:, :1], delta[:, :1])
+        # (the last MLP's partial sums cover all rows: final norm over all of them, logits of the text rows)
+        _, h = self._add_norm(delta, x, self.w["norm"])
+        return self.ops.linear(h[:, :1], self.lm_head)[..., : self.config.vocab_size]
 
     def _boundary_attention(self, qh, kh, vh, kc, vc, large, rows):
         """Attention and cache update of one layer at a chunk-boundary step with the fused operators
@@ -508,9 +532,7 @@ class KsaQwen3ForCausalLM:
                 attn = ops.decode(q.transpose(1, 2), cache.key_cache[li], cache.value_cache[li], a, e,
                                   self.scaling)
             else:
-                q, k, v = self._qkv(lw, h, sum_rows)
-                q, k, v = ops.pre_attention(q, k, v, lw["q_norm"], lw["k_norm"], cos, sin, cfg.rms_norm_eps)
-                self._blend_summary(lw, h, sum_rows, cos, sin, q, k, v)
+                q, k, v = self._boundary_qkv(lw, h, sum_rows, cos, sin)
                 qh, kh, vh = q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2)
                 if hasattr(ops, "decode_boundary") and cache.boundary_fits_one_piece(li):
                     # fused operators: the cache only does the bookkeeping and names the rows
@@ -532,17 +554,16 @@ class KsaQwen3ForCausalLM:
                     sum_out = ops.decode(qh[:, :, 1:], k_cs, v_cs, 0, k_cs.shape[2], self.scaling)
                     cache.update_summary(kh[:, :, 1:], vh[:, :, 1:], li)
                     attn = torch.cat([text_out, sum_out], dim=1)
-            # a text step hands both products straight to the next norm; a boundary step slices them
             if boundary:
-                x, h = self._add_norm(ops.linear(attn.reshape(b, ids.shape[1], -1), lw["o_proj"]), x,
+                x, h = self._add_norm(ops.linear(attn.reshape(b, ids.shape[1], -1), lw["o_proj"], defer=True), x,
                                       lw["post_attention_layernorm"])
-                delta = self._mlp(lw, h)
+                delta = self._mlp(lw, h, defer=True)
             else:
                 x, delta = self._post_attention(lw, attn.reshape(b, ids.shape[1], -1), x)
         cache.reset_chunk_counter()
         if not boundary:
             return self._logits(x, delta)
-        return self._logits(x[:, :1], delta[:, :1])
+        return self._boundary_logits(x, delta)
 
     # ---- decode through a HIP graph ----------------------------------------------------
     def _text_step_body(self, st, cache):
@@ -599,9 +620,7 @@ class KsaQwen3ForCausalLM:
             kind = 1 if cache.is_large_window[li] else 0
             kc, vc, mv = cache.key_cache[li], cache.value_cache[li], cache._move_rows
             x, h = self._add_norm(delta, x, lw["input_layernorm"])
-            q, k, v = self._qkv(lw, h, sum_rows)
-            q, k, v = ops.pre_attention(q, k, v, lw["q_norm"], lw["k_norm"], cos, sin, cfg.rms_norm_eps)
-            self._blend_summary(lw, h, sum_rows, cos, sin, q, k, v)
+            q, k, v = self._boundary_qkv(lw, h, sum_rows, cos, sin)
             qh, kh, vh = q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2)
             if hasattr(ops, "decode_boundary"):
                 rows = dict(text=bc[kind, 0], start=bc[kind, 1], end=bc[kind, 2])
@@ -626,10 +645,10 @@ class KsaQwen3ForCausalLM:
                     mv(vh[:, :, 1:], vc, S, dst_start_seq=bc[1, 3])
                     sum_out = ops.decode(qh[:, :, 1:], kc, vc, bc[1, 4], bc[1, 5], self.scaling)
                 attn = torch.cat([text_out, sum_out], dim=1)
-            x, h = self._add_norm(ops.linear(attn.reshape(b, 1 + S, -1), lw["o_proj"]), x,
+            x, h = self._add_norm(ops.linear(attn.reshape(b, 1 + S, -1), lw["o_proj"], defer=True), x,
                                   lw["post_attention_layernorm"])
-            delta = self._mlp(lw, h)
-        return self._logits(x[:, :1], delta[:, :1])
+            delta = self._mlp(lw, h, defer=True)
+        return self._boundary_logits(x, delta)
 
     def _stage_ints(self, st, key, vals):
         """Host integers `vals` (a flat list) -> the int32 device tensor st[key], through a ring of

@@ -80,7 +80,7 @@ def pre_attention_partials(qkv, Hq: int, Hkv: int, D: int, q_norm_weight: torch.
                            v_out: Optional[torch.Tensor] = None,
                            kv_out_row: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """`pre_attention` on a fused q | k | v projection [b, S, (Hq + 2 Hkv) D] that is still the
-    `SplitKPartials` of a deferred `linear_rows` (at most 16 rows): the partial sums are added
+    `SplitKPartials` of a deferred `linear_rows` (at most 128 rows): the partial sums are added
     inside the kernel, with the outputs of the two-kernel form."""
     from .gemm import SplitKPartials
     assert isinstance(qkv, SplitKPartials) and len(qkv.shape) == 3 and qkv.shape[-1] == (Hq + 2 * Hkv) * D

@@ -11,7 +11,12 @@ import torch
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("M,N,K", [(1, 16, 32), (8, 6144, 2560), (8, 2560, 4096), (8, 19456, 2560),
-                                   (8, 2560, 9728), (16, 1000, 640), (3, 40, 96), (5, 151936, 2560)])
+                                   (8, 2560, 9728), (16, 1000, 640), (3, 40, 96), (5, 151936, 2560),
+                                   # 17 to 128 rows: the wide form (row blocks of 16; K with a short last chunk;
+                                   # column tiles that end inside a wave's 16 columns)
+                                   (17, 16, 32), (72, 6144, 2560), (72, 2560, 4096), (72, 19456, 2560),
+                                   (72, 2560, 9728), (64, 1000, 640), (33, 40, 96), (128, 300, 1120),
+                                   (100, 2050, 544), (80, 151936, 2560), (112, 130, 1024)])
 def test_gpu_linear_rows(dtype, M, N, K):
     from ksa_amd.gemm import linear_rows
     g = torch.Generator().manual_seed(M * 7 + N + K)
@@ -36,7 +41,7 @@ def test_gpu_linear_rows_views_and_errors():
     ref = (x.double() @ w[64:128].double().T)
     assert y.shape == (2, 4, 64) and (y.double() - ref).abs().max() <= 0.02 * ref.abs().max()
     with pytest.raises(AssertionError):
-        linear_rows(torch.zeros(17, 64, dtype=torch.bfloat16, device="cuda"), w[:, :64].contiguous())
+        linear_rows(torch.zeros(129, 64, dtype=torch.bfloat16, device="cuda"), w[:, :64].contiguous())
     with pytest.raises(KsaError):
         linear_rows(torch.zeros(2, 48, dtype=torch.bfloat16, device="cuda"),
                     torch.zeros(8, 48, dtype=torch.bfloat16, device="cuda"))   # K not a multiple of 32
@@ -45,12 +50,14 @@ def test_gpu_linear_rows_views_and_errors():
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("M,N,K", [(8, 2560, 4096), (8, 2560, 9728), (1, 2560, 4096), (16, 1024, 1024), (3, 64, 512),
-                                   (2, 8192, 1024)])
+                                   (2, 8192, 1024), (72, 2560, 4096), (72, 2560, 9728), (40, 1024, 2048),
+                                   (128, 512, 4096)])
 def test_gpu_deferred_product_into_add_rmsnorm(dtype, M, N, K):
     """A product left as K-split partial sums and added inside `add_rmsnorm`: the sum with the
     residual is bit for bit what the reduced product followed by `add_rmsnorm` gives (same
     summation order over the splits, same rounding points); the normalised output may differ by
-    one unit in the last place in a few elements, because the mean square is summed over a
+    one unit in the last place of the rounded normalised value in a few elements (two of the product
+    with the weight when that falls into the binade below), because the mean square is summed over a
     workgroup instead of a wave.  A product that is not split comes back as a plain tensor."""
     from ksa_amd import add_rmsnorm
     from ksa_amd.gemm import SplitKPartials, linear_rows
@@ -68,13 +75,15 @@ def test_gpu_deferred_product_into_add_rmsnorm(dtype, M, N, K):
     a, b = h0.float().flatten(), h1.float().flatten()
     mant = 7 if dtype == torch.bfloat16 else 10
     ulp = torch.exp2(torch.floor(torch.log2(a.abs().clamp_min(2.0 ** -14))) - mant)
-    assert ((a - b).abs() <= ulp * 1.01).all()
+    assert ((a - b).abs() <= 2 * ulp * 1.001).all()
+    assert ((a - b).abs() > ulp * 1.01).float().mean() <= 1e-4
     assert (a != b).float().mean() <= 0.01
 
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("M,I,K", [(8, 9728, 2560), (1, 9728, 2560), (16, 520, 1024), (5, 64, 512)])
+@pytest.mark.parametrize("M,I,K", [(8, 9728, 2560), (1, 9728, 2560), (16, 520, 1024), (5, 64, 512), (72, 1024, 4096),
+                                   (30, 520, 2048)])
 def test_gpu_deferred_gate_up_into_silu_mul(dtype, M, I, K):
     """gate | up left as K-split partial sums and added inside `silu_mul`: bit for bit the
     two-kernel result (the halves are summed in split order and rounded before the activation)."""
@@ -96,7 +105,9 @@ def test_gpu_deferred_gate_up_into_silu_mul(dtype, M, I, K):
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("M,I,K", [(8, 9728, 2560), (1, 9728, 2560), (16, 520, 1024), (5, 64, 512), (3, 40, 96),
-                                   (8, 1000, 1056), (2, 48, 8192), (16, 32, 5088)])
+                                   (8, 1000, 1056), (2, 48, 8192), (16, 32, 5088),
+                                   # 17 to 128 rows: x in chunks through LDS, gate and up waves meet behind the walk
+                                   (72, 9728, 2560), (17, 40, 96), (64, 1000, 1056), (128, 200, 512), (100, 72, 1600)])
 def test_gpu_gate_up_silu_one_launch(dtype, M, I, K):
     """The gate | up projection with the activation folded in (one launch, K not split) against the
     fp64 statement of the same rounding points - out = round(SiLU(round(g))) * round(u) - and against
@@ -104,7 +115,10 @@ def test_gpu_gate_up_silu_one_launch(dtype, M, I, K):
     a gate or up value that lies next to a rounding boundary may round the other way: the result
     may then differ from the exact-sum statement by one unit in the last place of an intermediate
     (relative 2^-7 in bf16, 2^-10 in fp16), which SiLU passes on multiplied by |1 + g (1 - sigmoid(g))|
-    <= 1 + |g|, in a small share of the elements."""
+    <= 1 + |g|, in a small share of the elements.  Where a gate or up sum cancels to almost nothing the
+    fp32 sum itself is off by more than such a unit (about 1e-6 absolute at these magnitudes; the
+    two-kernel path shows the same): an absolute term of 2e-6 on either sum, passed on through the
+    other factor."""
     from ksa_amd import silu_mul
     from ksa_amd.gemm import gate_up_silu_rows, linear_rows
     g = torch.Generator().manual_seed(M + I + K)
@@ -117,7 +131,8 @@ def test_gpu_gate_up_silu_one_launch(dtype, M, I, K):
     want = ((gate / (1 + torch.exp(-gate))).to(dtype).double() * up).to(dtype)
     a, b = got[0].float().cpu(), want.float()
     ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
-    tol = ulp * (3 + gate.abs().float()) * b.abs() + 1e-6
+    act64 = gate / (1 + torch.exp(-gate))
+    tol = ulp * (3 + gate.abs().float()) * b.abs() + 1e-6 + 2e-6 * (1.1 * up.abs() + act64.abs()).float()
     assert ((a - b).abs() <= tol).all(), ((a - b).abs() / tol).max()
     assert (a != b).float().mean() <= 0.02
     two = silu_mul(linear_rows(x.cuda(), w.cuda()))

@@ -199,7 +199,8 @@ def test_pre_attention_rejects_bad_inputs():
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("b,S,Hq,Hkv,D", [(8, 1, 32, 8, 128), (1, 1, 32, 8, 128), (2, 3, 6, 2, 64), (16, 1, 4, 4, 128)])
+@pytest.mark.parametrize("b,S,Hq,Hkv,D", [(8, 1, 32, 8, 128), (1, 1, 32, 8, 128), (2, 3, 6, 2, 64), (16, 1, 4, 4, 128),
+                                          (8, 9, 32, 8, 128), (64, 1, 32, 8, 128), (14, 9, 6, 2, 64)])
 def test_pre_attention_gpu_from_split_k_partials(dtype, b, S, Hq, Hkv, D):
     """q | k | v still as the K-split partial sums of the fused projection: the kernel adds them
     itself and returns bit for bit what the reduced projection followed by `pre_attention` gives,
