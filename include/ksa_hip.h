@@ -207,9 +207,9 @@ int ksa_pre_attention(const void* q, const void* k, const void* v, const void* q
                       const int32_t* kv_out_row_seq, float eps, void* stream);
 
 /* ksa_pre_attention whose q | k | v rows are still the K-split partial sums of the fused qkv
- * projection (fp32 [ksplit][16][(Hq + 2 Hkv) D], left by ksa_gemm_rows called with out == NULL;
- * row = batch index * S + position): summed in split order and rounded first, so the outputs are
- * bit-identical to the two-kernel form.  batch * S <= 16. */
+ * projection (fp32 [ksplit][R][(Hq + 2 Hkv) D], R = batch * S rounded up to a multiple of 16, left by
+ * ksa_gemm_rows called with out == NULL; row = batch index * S + position): summed in split order and
+ * rounded first, so the outputs are bit-identical to the two-kernel form.  batch * S <= 128. */
 int ksa_pre_attention_partials(const float* partials, int ksplit, const void* q_weight,
                                const void* k_weight, const void* cos, const void* sin, void* q_out,
                                void* k_out, void* v_out, int batch, int S, int Hq, int Hkv, int D,
@@ -230,11 +230,12 @@ int ksa_add_rmsnorm(const void* x, const void* residual, const void* weight, voi
                     long long sum_row_stride, int dtype, float eps, void* stream);
 
 /* ksa_add_rmsnorm whose x is not a tensor yet but the K-split partial sums that ksa_gemm_rows
- * leaves in its workspace when called with out == NULL (fp32 [ksplit][16][H]): x = the sum over
+ * leaves in its workspace when called with out == NULL (fp32 [ksplit][R][H], R = rows rounded up to a
+ * multiple of 16): x = the sum over
  * the splits in split order, rounded to the 16-bit type.  out_sum is bit-identical to
  * ksa_gemm_rows with an output followed by ksa_add_rmsnorm; out_norm agrees to one unit in the
  * last place (the mean square is summed in a different order).  One launch less per o_proj /
- * down_proj -> residual add + norm (HF:944-952).  rows <= 16, H <= 8192; residual and out_sum
+ * down_proj -> residual add + norm (HF:944-952).  rows <= 128, H <= 8192; residual and out_sum
  * are required. */
 int ksa_add_rmsnorm_partials(const float* partials, int ksplit, const void* residual,
                              const void* weight, void* out_norm, void* out_sum, int rows, int H,
@@ -257,37 +258,44 @@ int ksa_argmax_rows(const void* x, long long* out, int rows, int N, long long x_
                     void* stream);
 
 /* ksa_silu_mul whose gate | up is still the K-split partial sums of the fused gate_up projection
- * (fp32 [ksplit][16][2 I], left by ksa_gemm_rows called with out == NULL): both halves are summed
- * in split order and rounded first, so the result is bit-identical to the two-kernel form.
- * rows <= 16. */
+ * (fp32 [ksplit][R][2 I], R = rows rounded up to a multiple of 16, left by ksa_gemm_rows called with
+ * out == NULL): both halves are summed in split order and rounded first, so the result is bit-identical
+ * to the two-kernel form.  rows <= 128. */
 int ksa_silu_mul_partials(const float* partials, int ksplit, void* out, int rows, int I,
                           long long out_row_stride, int dtype, void* stream);
 
-/* y = x W^T for at most 16 rows of x (decode steps), bound by the weight bytes.
+/* y = x W^T for at most 128 rows of x (decode steps), bound by the weight bytes.
  * Replaces torch.nn.functional.linear at the projections of a decode step (HF:628-641 q/k/v and
  * o projections, HF:507-514 MLP, HF:1338 lm_head), bias-free as in the reference's config.
  *   x [M, K], w [N, K], out [M, N], 16-bit, row strides in elements (x, w: multiples of 8);
  *   K a multiple of 32; fp32 accumulation, one rounding at the end.
- * ksplit > 1 splits K over workgroups (ksa_gemm_rows_auto_splits) and needs
- * ksa_gemm_rows_workspace_bytes(N, ksplit) bytes of device workspace.  With ksplit > 1 out may
- * be NULL: the partial sums (fp32 [ksplit][16][N]) are then left in the workspace for a consumer
- * that adds them itself (ksa_add_rmsnorm_partials, ksa_silu_mul_partials,
- * ksa_pre_attention_partials). */
+ * ksplit > 1 splits K over workgroups and needs a device workspace for the partial sums:
+ * ksa_gemm_rows_splits(M, N, K) gives the split count to use and ksa_gemm_rows_partials_bytes(M, N,
+ * ksplit) the bytes (ksa_gemm_rows_auto_splits(N, K) and ksa_gemm_rows_workspace_bytes(N, ksplit) are
+ * the same answers for M <= 16).  For M > 16 (a kernel of its own: every weight fragment meets each
+ * 16-row block of x, staged through LDS in chunks of 512 elements of K) only split counts that
+ * ksa_gemm_rows_splits can return are taken - slices are whole chunks, none empty - anything else is
+ * KSA_ERR_INVALID.  With ksplit > 1 out may be NULL: the partial sums (fp32 [ksplit][R][N], R = M
+ * rounded up to a multiple of 16) are then left in the workspace for a consumer that adds them itself
+ * (ksa_add_rmsnorm_partials, ksa_silu_mul_partials, ksa_pre_attention_partials). */
 int ksa_gemm_rows_auto_splits(int N, int K);
 size_t ksa_gemm_rows_workspace_bytes(int N, int ksplit);
+int ksa_gemm_rows_splits(int M, int N, int K);
+size_t ksa_gemm_rows_partials_bytes(int M, int N, int ksplit);
 int ksa_gemm_rows(const void* x, const void* w, void* out, int M, int N, int K, long long x_row_stride,
                   long long w_row_stride, long long out_row_stride, int dtype, int ksplit,
                   void* workspace, size_t workspace_bytes, void* stream);
 
-/* The MLP's gate | up projection with its activation folded in, for at most 16 rows of x:
+/* The MLP's gate | up projection with its activation folded in, for at most 128 rows of x:
  * out = round(SiLU(round(x w_gate^T))) * round(x w_up^T), one launch, no partial sums in memory.
  * Replaces act_fn(gate_proj(x)) * up_proj(x) of Qwen3MLP.forward (HF:507-514) at a decode step, i.e.
  * ksa_gemm_rows on the fused gate | up matrix followed by ksa_silu_mul (same rounding points; the
  * fp32 sums run over K in one chain instead of split-K order, so the 16-bit results can differ from
  * that pair's in the last place).
  *   x [M, K], w [2 I, K] (gate rows, then up rows), out [M, I]; K a multiple of 32; row strides in
- *   elements (x, w: multiples of 8).  x is held in LDS whole: M (K + 8) 2 bytes beyond 160 KiB are
- *   KSA_ERR_UNSUPPORTED (use ksa_gemm_rows and ksa_silu_mul then). */
+ *   elements (x, w: multiples of 8).  Up to 16 rows x is held in LDS whole: M (K + 8) 2 bytes beyond
+ *   160 KiB are KSA_ERR_UNSUPPORTED (use ksa_gemm_rows and ksa_silu_mul then); 17 to 128 rows go
+ *   through LDS in chunks (any K), half of a workgroup's waves on gate columns, half on up columns. */
 int ksa_gemm_rows_gate_up_silu(const void* x, const void* w, void* out, int M, int I, int K,
                                long long x_row_stride, long long w_row_stride, long long out_row_stride,
                                int dtype, void* stream);
