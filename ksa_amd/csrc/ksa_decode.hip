@@ -99,13 +99,22 @@ __global__ __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) void ksa_decode_kerne
     const int lh = lane >> 5;
 
     const int split = blockIdx.x;
-    const int colblk = blockIdx.y / p.Hkv;
     const int kvh = blockIdx.y % p.Hkv;
     const int bz = blockIdx.z;
 
     uint16_t* Kw = reinterpret_cast<uint16_t*>(smem) + wave * kStage;
     uint16_t* Vw = Kw + kRows * KROW;
 
+    // One column block per workgroup - except in the chunk-boundary form, where the workgroup of the text
+    // token's block takes the summary tokens' blocks behind it (their row range is one chunk: a tile or two
+    // for two of the splits, nothing for the others).  As workgroups of their own, scattered between the long
+    // ones, those short blocks held places of a CU for a chain of memory round trips under full load, and the
+    // long workgroups that had to wait for the places ended late: +8 us per small-window layer and +27 us
+    // per large-window layer of a boundary step.
+    const int colblk_first = p.split_q ? 0 : blockIdx.y / p.Hkv;
+    const int colblk_last = p.split_q ? p.ncols_pad / 32 - 1 : colblk_first;
+    for (int colblk = colblk_first; colblk <= colblk_last; ++colblk) {
+    if (colblk != colblk_first) __syncthreads();  // the previous block's merge area becomes staging again
     const bool second = p.split_q && colblk > 0;  // the summary tokens' columns and their own row range
     const int r_begin = second ? (p.start2 ? p.start2[bz] : p.start20) : (p.start ? p.start[bz] : p.start0);
     const int r_end = second ? (p.end2 ? p.end2[bz] : p.end20) : (p.end ? p.end[bz] : p.end0);
@@ -115,6 +124,19 @@ __global__ __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) void ksa_decode_kerne
                     (kWaves * kRows);
     const int s0 = r_begin + split * per;
     const int s1 = min(r_end, s0 + per);
+
+    if (p.nsplit > 1 && s0 >= s1) {
+        // an empty slice (a short range: the summary tokens' chunk at a boundary step, a sequence with few
+        // rows): the merge only needs to know that there is nothing here (it does not read the sums then)
+        const int ncol = !p.split_q ? min(32, p.ncols - colblk * 32)
+                                    : (colblk == 0 ? p.g : min(32, (p.Q - 1) * p.g - (colblk - 1) * 32));
+        if (tid < ncol) {
+            const int64_t slot = (((int64_t)bz * p.Hkv + kvh) * p.nsplit + split) * p.ncols_pad + colblk * 32 + tid;
+            p.ws_ml[slot * 2] = -INFINITY;
+            p.ws_ml[slot * 2 + 1] = 0.f;
+        }
+        continue;
+    }
 
     // column (query token qi, head gi of the group) owned by this lane
     int qi, gi;
@@ -276,6 +298,7 @@ __global__ __launch_bounds__(kThreads, (D <= 128 ? 2 : 1)) void ksa_decode_kerne
             }
         }
     }
+    }  // column blocks of this workgroup
 }
 
 // second stage: merge the splits of one (sequence, kv head, column)
@@ -310,9 +333,11 @@ __global__ __launch_bounds__(D) void ksa_decode_merge_kernel(const DecodeParams 
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
             if (s0 + u < p.nsplit) {
-                const float f = (m[u] == -INFINITY) ? 0.f : ksa_exp2(m[u] - mx);
-                acc += o[u] * f;
-                l += ls[u] * f;
+                // (an empty slice leaves its sums unwritten: nothing of it may enter, not even times zero)
+                const bool some = m[u] != -INFINITY;
+                const float f = some ? ksa_exp2(m[u] - mx) : 0.f;
+                acc = some ? fmaf(o[u], f, acc) : acc;
+                l = some ? fmaf(ls[u], f, l) : l;
             }
         }
     }
@@ -323,7 +348,7 @@ __global__ __launch_bounds__(D) void ksa_decode_merge_kernel(const DecodeParams 
 
 template <typename T, int D>
 int launch(const DecodeParams& p, int batch, hipStream_t stream) {
-    const int colblks = p.ncols_pad / 32;
+    const int colblks = p.split_q ? 1 : p.ncols_pad / 32;  // (boundary form: a workgroup walks its column blocks)
     dim3 grid(p.nsplit, p.Hkv * colblks, batch);
     hipLaunchKernelGGL((ksa_decode_kernel<T, D>), grid, dim3(kThreads), 0, stream, p);
     if (p.nsplit > 1) {
