@@ -197,14 +197,18 @@ int ksa_copy_rows_multi(int n_moves, const void* const* src, void* const* dst,
  *   kv_out_row_seq: NULL, or int32 [batch] in device memory: sequence b's k and v go
  *   kv_out_row_seq[b] rows (of k_out_strides[1] / v_out_strides[1]) further down - the cache
  *   cursor of update_text (HF:306-336) when only the device knows it (graph replay); the
- *   caller guarantees the rows exist. */
+ *   caller guarantees the rows exist.  With kv_out_row_per_token != 0 the array is int32
+ *   [batch][S] and names the destination row of every token's k and v outright, in place of its
+ *   position: the text token and the summary tokens of a chunk-boundary step go to different
+ *   places of the cache (update_text and the scratch rows of update_summary, HF:306-398). */
 int ksa_pre_attention(const void* q, const void* k, const void* v, const void* q_weight,
                       const void* k_weight, const void* cos, const void* sin, void* q_out,
                       void* k_out, void* v_out, int batch, int S, int Hq, int Hkv, int D, int dtype,
                       const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
                       const int64_t* q_out_strides, const int64_t* k_out_strides,
                       const int64_t* v_out_strides, const int64_t* cos_strides,
-                      const int32_t* kv_out_row_seq, float eps, void* stream);
+                      const int32_t* kv_out_row_seq, int kv_out_row_per_token, float eps,
+                      void* stream);
 
 /* ksa_pre_attention whose q | k | v rows are still the K-split partial sums of the fused qkv
  * projection (fp32 [ksplit][R][(Hq + 2 Hkv) D], R = batch * S rounded up to a multiple of 16, left by
@@ -215,7 +219,8 @@ int ksa_pre_attention_partials(const float* partials, int ksplit, const void* q_
                                void* k_out, void* v_out, int batch, int S, int Hq, int Hkv, int D,
                                int dtype, const int64_t* q_out_strides, const int64_t* k_out_strides,
                                const int64_t* v_out_strides, const int64_t* cos_strides,
-                               const int32_t* kv_out_row_seq, float eps, void* stream);
+                               const int32_t* kv_out_row_seq, int kv_out_row_per_token, float eps,
+                      void* stream);
 
 /* Residual add + RMSNorm over the hidden size, one pass.
  * Replaces Qwen3RMSNorm.forward (HF:64-79: fp32 normalisation, rounded to the 16-bit type, times

@@ -37,9 +37,9 @@ _SIGNATURES = {
                                 + [ctypes.c_float, _int, _vp, ctypes.c_size_t, _vp]),
     "ksa_copy_rows_multi": (_int, [_int, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _vp, _vp, _vp]),
     "ksa_copy_rows": (_int, [_vp] * 4 + [_int] * 6 + [_i64p] * 2 + [_vp]),
-    "ksa_pre_attention": (_int, [_vp] * 10 + [_int] * 6 + [_i64p] * 7 + [_vp, ctypes.c_float, _vp]),
+    "ksa_pre_attention": (_int, [_vp] * 10 + [_int] * 6 + [_i64p] * 7 + [_vp, _int, ctypes.c_float, _vp]),
     "ksa_pre_attention_partials": (_int, [_vp, _int] + [_vp] * 7 + [_int] * 6 + [_i64p] * 4
-                                   + [_vp, ctypes.c_float, _vp]),
+                                   + [_vp, _int, ctypes.c_float, _vp]),
     "ksa_add_rmsnorm": (_int, [_vp] * 5 + [ctypes.c_longlong, _int] + [ctypes.c_longlong] * 4
                         + [_int, ctypes.c_float, _vp]),
     "ksa_add_rmsnorm_partials": (_int, [_vp, _int] + [_vp] * 4 + [_int, _int] + [ctypes.c_longlong] * 3

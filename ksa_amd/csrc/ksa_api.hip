@@ -3,7 +3,7 @@
 
 #include "ksa_api_internal.h"
 
-extern "C" int ksa_version(void) { return 101; }
+extern "C" int ksa_version(void) { return 102; }
 
 extern "C" const char* ksa_error_string(int code) {
     switch (code) {

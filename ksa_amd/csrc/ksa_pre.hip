@@ -28,7 +28,8 @@ struct PreParams {
     const uint16_t* src[3];   // q, k, v projections  [batch, S, H, D] by strides
     uint16_t* dst[3];         // q, k, v outputs
     const uint16_t* w[2];     // q_norm, k_norm weights [D]
-    const int32_t* kv_row;    // [batch] or null: row added to the k / v destination of a sequence
+    const int32_t* kv_row;    // null, or [batch]: row added to the k / v destination of a sequence, or
+    int kv_row_per_token;     // (flag) [batch][S]: the k / v destination row of every token, in place of its position
     const float* part;        // if set: q | k | v rows as K-split partial sums [ksplit][ksa_partial_rows(batch S)][(Hq + 2 Hkv) D], src unused
     int ksplit;
     const uint16_t* cos;      // [batch or 1, S, D]
@@ -157,7 +158,8 @@ __global__ __launch_bounds__(256) void ksa_pre_attention_kernel(const PreParams 
         g.col0 = ((g.which == 0 ? 0 : (g.which == 1 ? p.Hq : p.Hq + p.Hkv)) + g.h0) * D;
         g.sbase = p.src[g.which] + nb * p.s_bs[g.which] + (int64_t)ns * p.s_rs[g.which] + (int64_t)g.h0 * p.s_hs[g.which];
         // (k and v may go to a row of their sequence that the host does not know: a cache cursor)
-        const int64_t drow = ns + ((g.which != 0 && p.kv_row) ? p.kv_row[nb] : 0);
+        int64_t drow = ns;
+        if (g.which != 0 && p.kv_row) drow = p.kv_row_per_token ? p.kv_row[g.tok] : ns + p.kv_row[nb];
         g.dbase = p.dst[g.which] + nb * p.d_bs[g.which] + drow * p.d_rs[g.which] + (int64_t)g.h0 * p.d_hs[g.which];
         gi += gstep;
         return g;
@@ -290,8 +292,8 @@ extern "C" int ksa_pre_attention(const void* q, const void* k, const void* v, co
                                  int dtype, const int64_t* q_strides, const int64_t* k_strides,
                                  const int64_t* v_strides, const int64_t* q_out_strides,
                                  const int64_t* k_out_strides, const int64_t* v_out_strides,
-                                 const int64_t* cos_strides, const int32_t* kv_out_row_seq, float eps,
-                                 void* stream) {
+                                 const int64_t* cos_strides, const int32_t* kv_out_row_seq, int kv_out_row_per_token,
+                                 float eps, void* stream) {
     if (!q || !k || !v || !q_weight || !k_weight || !cos || !sin || !q_out || !k_out || !v_out)
         return KSA_ERR_NULL;
     if (!q_strides || !k_strides || !v_strides || !q_out_strides || !k_out_strides || !v_out_strides ||
@@ -319,6 +321,7 @@ extern "C" int ksa_pre_attention(const void* q, const void* k, const void* v, co
     p.w[0] = (const uint16_t*)q_weight, p.w[1] = (const uint16_t*)k_weight;
     p.cos = (const uint16_t*)cos, p.sin = (const uint16_t*)sin;
     p.kv_row = kv_out_row_seq;
+    p.kv_row_per_token = kv_out_row_per_token != 0;
     const int64_t* in[] = {q_strides, k_strides, v_strides};
     const int64_t* out[] = {q_out_strides, k_out_strides, v_out_strides};
     for (int i = 0; i < 3; ++i) {
@@ -336,7 +339,8 @@ extern "C" int ksa_pre_attention_partials(const float* partials, int ksplit, con
                                           void* k_out, void* v_out, int batch, int S, int Hq, int Hkv, int D,
                                           int dtype, const int64_t* q_out_strides, const int64_t* k_out_strides,
                                           const int64_t* v_out_strides, const int64_t* cos_strides,
-                                          const int32_t* kv_out_row_seq, float eps, void* stream) {
+                                          const int32_t* kv_out_row_seq, int kv_out_row_per_token, float eps,
+                                          void* stream) {
     if (!partials || !q_weight || !k_weight || !cos || !sin || !q_out || !k_out || !v_out) return KSA_ERR_NULL;
     if (!q_out_strides || !k_out_strides || !v_out_strides || !cos_strides) return KSA_ERR_NULL;
     if (batch <= 0 || S <= 0 || (int64_t)batch * S > kMaxPartialRows || Hq <= 0 || Hkv <= 0 || ksplit < 1 || ksplit > 64 ||
@@ -360,6 +364,7 @@ extern "C" int ksa_pre_attention_partials(const float* partials, int ksplit, con
     p.w[0] = (const uint16_t*)q_weight, p.w[1] = (const uint16_t*)k_weight;
     p.cos = (const uint16_t*)cos, p.sin = (const uint16_t*)sin;
     p.kv_row = kv_out_row_seq;
+    p.kv_row_per_token = kv_out_row_per_token != 0;
     const int64_t* out[] = {q_out_strides, k_out_strides, v_out_strides};
     for (int i = 0; i < 3; ++i) {
         p.s_hs[i] = D;  // (only the lane offsets are derived from it; the source is `partials`)

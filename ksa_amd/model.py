@@ -322,19 +322,48 @@ class KsaQwen3ForCausalLM:
             return self.ops.add_rmsnorm(x, None, w, self.config.rms_norm_eps)
         return self.ops.add_rmsnorm(delta, x, w, self.config.rms_norm_eps)
 
-    def _boundary_qkv(self, lw, h, sum_rows, cos, sin):
+    def _boundary_rows_in_cache(self):
+        """Whether a boundary step may write the new K/V rows straight to their cache rows (a row per token,
+        `pre_attention(..., kv_out_row=[b, 1 + S])`): the fused operators, and no second set of summary
+        projections whose rows are blended in after the pre-attention step."""
+        return (hasattr(self.ops, "decode_boundary") and hasattr(self.ops, "pre_attention_partials")
+                and not self.config.summary_independent_parameters)
+
+    def _boundary_row_table(self, text, base, b):
+        """int32 [b, 1 + S] on the device: the cache row of every token of a boundary step - the text token's
+        row `text`, summary token i at `base + i`; `text` / `base` ints or int32 device tensors [b]."""
+        S = self.config.summary_token_num
+        if not torch.is_tensor(text) and not torch.is_tensor(base):
+            row = [int(text)] + [int(base) + i for i in range(S)]
+            return torch.tensor([row] * b, dtype=torch.int32).to(self.device)
+        # (no host-to-device copies: this runs inside a recording)
+        some = text if torch.is_tensor(text) else base
+        as_rows = lambda v: v.to(torch.int32).expand(b) if torch.is_tensor(v) else torch.full_like(some, int(v), dtype=torch.int32).expand(b)
+        ar = torch.arange(S, dtype=torch.int32, device=self.device)
+        return torch.cat([as_rows(text)[:, None], as_rows(base)[:, None] + ar[None]], dim=1).contiguous()
+
+    def _boundary_qkv(self, lw, h, sum_rows, cos, sin, slots=None):
         """q, k, v [b, 1 + S, H, D] (normalised, rotated) of a chunk-boundary step's rows.  With one
         set of projection weights the product may stay the K-split partial sums of the few-rows GEMM,
-        which the pre-attention kernel adds itself (one launch less)."""
+        which the pre-attention kernel adds itself (one launch less).  `slots` = (key cache, value cache,
+        row table of `_boundary_row_table`): k and v go straight to those cache rows and are not returned."""
         cfg, ops = self.config, self.ops
+        out = {}
+        if slots is not None:
+            kc, vc, table = slots
+            n = table.shape[1]
+            out = dict(k_out=kc[:, :, :n].transpose(1, 2), v_out=vc[:, :, :n].transpose(1, 2), kv_out_row=table)
         qkv = None
         if not cfg.summary_independent_parameters and hasattr(ops, "pre_attention_partials"):
             qkv = ops.linear(h, lw["qkv_proj"], defer=True)
         if qkv is not None and not torch.is_tensor(qkv):
-            return ops.pre_attention_partials(qkv, cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim,
-                                              lw["q_norm"], lw["k_norm"], cos, sin, cfg.rms_norm_eps)
+            q, k, v = ops.pre_attention_partials(qkv, cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim,
+                                                 lw["q_norm"], lw["k_norm"], cos, sin, cfg.rms_norm_eps, **out)
+            return (q, None, None) if slots is not None else (q, k, v)
         q, k, v = self._split_qkv(qkv) if qkv is not None else self._qkv(lw, h, sum_rows)
-        q, k, v = ops.pre_attention(q, k, v, lw["q_norm"], lw["k_norm"], cos, sin, cfg.rms_norm_eps)
+        q, k, v = ops.pre_attention(q, k, v, lw["q_norm"], lw["k_norm"], cos, sin, cfg.rms_norm_eps, **out)
+        if slots is not None:
+            return q, None, None
         self._blend_summary(lw, h, sum_rows, cos, sin, q, k, v)
         return q, k, v
 
@@ -354,24 +383,33 @@ class KsaQwen3ForCausalLM:
         qh [b, Hq, 1 + S, D], kh, vh [b, Hkv, 1 + S, D]; `rows` names the cache rows as
         `Qwen3RingBufferCache.boundary_slots` does, every value an int or an int32 device tensor [b]:
         small window: text, start, end, flush_src, flush_dst, flush_rows, append; large window: text,
-        start, end, spare, sum_start, sum_end (= spare - C, spare + S).  Returns [b, 1 + S, Hq, D]."""
+        start, end, spare, sum_start, sum_end (= spare - C, spare + S).  Returns [b, 1 + S, Hq, D].
+        kh, vh None: the pre-attention step has already written the step's K/V rows to the cache (text
+        row, scratch rows of a small window / spare rows of a large one), which leaves two launches
+        (+ the merge)."""
         ops = self.ops
         C, S = self.config.summary_chunk_size, self.config.summary_token_num
-        kt, vt, ks, vs = kh[:, :, :1], vh[:, :, :1], kh[:, :, 1:], vh[:, :, 1:]
+        in_cache = kh is None
+        if not in_cache:
+            kt, vt, ks, vs = kh[:, :, :1], vh[:, :, :1], kh[:, :, 1:], vh[:, :, 1:]
         if large:
             # the summary rows sit in spare rows behind the text for the length of the step, so that
             # [chunk text | own summaries] is one row range
             sp = rows["spare"]
-            ops.move_rows_multi([(kt, kc, 1, 0, rows["text"]), (vt, vc, 1, 0, rows["text"]),
-                                 (ks, kc, S, 0, sp), (vs, vc, S, 0, sp)])
+            if not in_cache:
+                ops.move_rows_multi([(kt, kc, 1, 0, rows["text"]), (vt, vc, 1, 0, rows["text"]),
+                                     (ks, kc, S, 0, sp), (vs, vc, S, 0, sp)])
             return ops.decode_boundary(qh, kc, vc, rows["start"], rows["end"], rows["sum_start"], rows["sum_end"],
                                        self.scaling)
-        ops.move_rows_multi([(kt, kc, 1, 0, rows["text"]), (vt, vc, 1, 0, rows["text"]),
-                             (ks, kc, S, 0, 0), (vs, vc, S, 0, 0)])
+        if not in_cache:
+            ops.move_rows_multi([(kt, kc, 1, 0, rows["text"]), (vt, vc, 1, 0, rows["text"]),
+                                 (ks, kc, S, 0, 0), (vs, vc, S, 0, 0)])
         attn = ops.decode_boundary(qh, kc, vc, rows["start"], rows["end"], 0, S + C, self.scaling)
+        # (the summaries are appended from the scratch rows when they did not come as tensors)
         ops.move_rows_multi([(kc, kc, rows["flush_rows"], rows["flush_src"], rows["flush_dst"]),
                              (vc, vc, rows["flush_rows"], rows["flush_src"], rows["flush_dst"]),
-                             (ks, kc, S, 0, rows["append"]), (vs, vc, S, 0, rows["append"])])
+                             (kc if in_cache else ks, kc, S, 0, rows["append"]),
+                             (vc if in_cache else vs, vc, S, 0, rows["append"])])
         return attn
 
     def _post_attention(self, lw, attn, x):
@@ -515,6 +553,7 @@ class KsaQwen3ForCausalLM:
         cos, sin = self._rope_tables(pos)
         x = self.w["embed_tokens"][ids]
         delta = None
+        tables = {}   # boundary step: (text row, first summary row) -> row table on the device
         for li, lw in enumerate(self.w["layers"]):
             x, h = self._add_norm(delta, x, lw["input_layernorm"])
             if not boundary:
@@ -532,9 +571,8 @@ class KsaQwen3ForCausalLM:
                 attn = ops.decode(q.transpose(1, 2), cache.key_cache[li], cache.value_cache[li], a, e,
                                   self.scaling)
             else:
-                q, k, v = self._boundary_qkv(lw, h, sum_rows, cos, sin)
-                qh, kh, vh = q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2)
-                if hasattr(ops, "decode_boundary") and cache.boundary_fits_one_piece(li):
+                fused = hasattr(ops, "decode_boundary") and cache.boundary_fits_one_piece(li)
+                if fused:
                     # fused operators: the cache only does the bookkeeping and names the rows
                     sl = cache.boundary_slots(li, S)
                     rows = dict(text=sl["text"], start=sl["attend"][0], end=sl["attend"][1])
@@ -543,6 +581,16 @@ class KsaQwen3ForCausalLM:
                     else:
                         rows.update(flush_src=sl["flush_src"], flush_dst=sl["flush_dst"],
                                     flush_rows=sl["flush_rows"], append=sl["append"])
+                slots = None
+                if fused and self._boundary_rows_in_cache():
+                    key = (rows["text"], rows["spare"] if cache.is_large_window[li] else 0)
+                    if key not in tables:  # the same for every layer of a kind: two small copies per step
+                        tables[key] = self._boundary_row_table(key[0], key[1], b)
+                    slots = (cache.key_cache[li], cache.value_cache[li], tables[key])
+                q, k, v = self._boundary_qkv(lw, h, sum_rows, cos, sin, slots)
+                qh = q.transpose(1, 2)
+                kh, vh = (None, None) if k is None else (k.transpose(1, 2), v.transpose(1, 2))
+                if fused:
                     attn = self._boundary_attention(qh, kh, vh, cache.key_cache[li], cache.value_cache[li],
                                                     cache.is_large_window[li], rows)
                 else:   # the reference's own sequence of cache calls
@@ -616,12 +664,16 @@ class KsaQwen3ForCausalLM:
         cos, sin = self._rope_tables(st["bpos"])
         x = self.w["embed_tokens"][ids]
         delta = None
+        tables = None
+        if self._boundary_rows_in_cache():  # where the step's K/V rows go: small window, large window
+            tables = (self._boundary_row_table(bc[0, 0], 0, b), self._boundary_row_table(bc[1, 0], bc[1, 3], b))
         for li, lw in enumerate(self.w["layers"]):
             kind = 1 if cache.is_large_window[li] else 0
             kc, vc, mv = cache.key_cache[li], cache.value_cache[li], cache._move_rows
             x, h = self._add_norm(delta, x, lw["input_layernorm"])
-            q, k, v = self._boundary_qkv(lw, h, sum_rows, cos, sin)
-            qh, kh, vh = q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2)
+            q, k, v = self._boundary_qkv(lw, h, sum_rows, cos, sin, None if tables is None else (kc, vc, tables[kind]))
+            qh = q.transpose(1, 2)
+            kh, vh = (None, None) if k is None else (k.transpose(1, 2), v.transpose(1, 2))
             if hasattr(ops, "decode_boundary"):
                 rows = dict(text=bc[kind, 0], start=bc[kind, 1], end=bc[kind, 2])
                 if kind:

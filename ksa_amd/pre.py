@@ -35,7 +35,9 @@ def pre_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q_norm_weig
     `cache_k[:, :, start:start + S].transpose(1, 2)` to write the keys straight into a
     [b, Hkv, capacity, D] cache tensor; they may alias the inputs.  `kv_out_row` (int32 [b] on
     the GPU) moves sequence b's k and v `kv_out_row[b]` rows further down their outputs: the
-    cache cursor when only the device knows it (a recorded step that is replayed).
+    cache cursor when only the device knows it (a recorded step that is replayed).  As int32
+    [b, S] it names the output row of every token's k and v outright (k_out / v_out then only give
+    the base address and the strides: pass the view that starts at row 0).
     """
     assert q.dtype in _DT and k.dtype == q.dtype and v.dtype == q.dtype, "q, k, v must share bf16 or fp16"
     assert q.is_cuda and k.is_cuda and v.is_cuda, "inputs must be on a GPU"
@@ -59,9 +61,10 @@ def pre_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q_norm_weig
         outs.append(given)
     qo, ko, vo = outs
     if kv_out_row is not None:
-        assert kv_out_row.is_cuda and kv_out_row.dtype == torch.int32 and kv_out_row.shape == (b,) \
-            and kv_out_row.is_contiguous(), "kv_out_row must be a contiguous int32 [b] GPU tensor"
+        assert kv_out_row.is_cuda and kv_out_row.dtype == torch.int32 and tuple(kv_out_row.shape) in ((b,), (b, S)) \
+            and kv_out_row.is_contiguous(), "kv_out_row must be a contiguous int32 [b] or [b, S] GPU tensor"
         assert k_out is not None and v_out is not None, "kv_out_row needs k_out and v_out"
+    per_token = int(kv_out_row is not None and kv_out_row.dim() == 2)
     cstr = (ctypes.c_int64 * 3)(cos.stride(0) if cos.shape[0] > 1 else 0, cos.stride(1), 0)
     L = _lib.lib()
     with torch.cuda.device(q.device):
@@ -69,7 +72,7 @@ def pre_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q_norm_weig
                                  cos.data_ptr(), sin.data_ptr(), qo.data_ptr(), ko.data_ptr(), vo.data_ptr(),
                                  b, S, Hq, Hkv, D, _DT[q.dtype], _bsh(q), _bsh(k), _bsh(v), _bsh(qo),
                                  _bsh(ko), _bsh(vo), cstr, None if kv_out_row is None else kv_out_row.data_ptr(),
-                                 float(eps), _lib.stream_ptr(q.device))
+                                 per_token, float(eps), _lib.stream_ptr(q.device))
     _lib.check(rc, "ksa_pre_attention")
     return qo, ko, vo
 
@@ -102,9 +105,10 @@ def pre_attention_partials(qkv, Hq: int, Hkv: int, D: int, q_norm_weight: torch.
         outs.append(given)
     qo, ko, vo = outs
     if kv_out_row is not None:
-        assert kv_out_row.is_cuda and kv_out_row.dtype == torch.int32 and kv_out_row.shape == (b,) \
-            and kv_out_row.is_contiguous(), "kv_out_row must be a contiguous int32 [b] GPU tensor"
+        assert kv_out_row.is_cuda and kv_out_row.dtype == torch.int32 and tuple(kv_out_row.shape) in ((b,), (b, S)) \
+            and kv_out_row.is_contiguous(), "kv_out_row must be a contiguous int32 [b] or [b, S] GPU tensor"
         assert k_out is not None and v_out is not None, "kv_out_row needs k_out and v_out"
+    per_token = int(kv_out_row is not None and kv_out_row.dim() == 2)
     cstr = (ctypes.c_int64 * 3)(cos.stride(0) if cos.shape[0] > 1 else 0, cos.stride(1), 0)
     L = _lib.lib()
     with torch.cuda.device(dev):
@@ -112,6 +116,6 @@ def pre_attention_partials(qkv, Hq: int, Hkv: int, D: int, q_norm_weight: torch.
                                           cos.data_ptr(), sin.data_ptr(), qo.data_ptr(), ko.data_ptr(),
                                           vo.data_ptr(), b, S, Hq, Hkv, D, _DT[dtype], _bsh(qo), _bsh(ko),
                                           _bsh(vo), cstr, None if kv_out_row is None else kv_out_row.data_ptr(),
-                                          float(eps), _lib.stream_ptr(dev))
+                                          per_token, float(eps), _lib.stream_ptr(dev))
     _lib.check(rc, "ksa_pre_attention_partials")
     return qo, ko, vo

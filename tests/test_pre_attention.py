@@ -238,3 +238,57 @@ def test_pre_attention_gpu_from_split_k_partials(dtype, b, S, Hq, Hkv, D):
         r = int(cursor[i])
         assert torch.equal(kc[i, :, r:r + S].transpose(0, 1), k0[i])
         assert torch.equal(vc[i, :, r:r + S].transpose(0, 1), v0[i])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("from_partials", [False, True])
+@pytest.mark.parametrize("b,S,Hq,Hkv,D", [(8, 9, 32, 8, 128), (3, 5, 6, 2, 64)])
+def test_pre_attention_gpu_row_per_token(from_partials, b, S, Hq, Hkv, D):
+    """`kv_out_row` as a table [b, S]: every token's k and v land in the cache row the table names (a
+    chunk-boundary step: the text token at the cache cursor, the summary tokens in rows of their own),
+    bit for bit the values of the plain call; q is unchanged; no other cache row is touched."""
+    import ksa_amd
+    from ksa_amd.gemm import SplitKPartials, linear_rows
+    from ksa_amd.pre import pre_attention_partials
+    dev = torch.device("cuda")
+    dtype = torch.bfloat16
+    K = 2560
+    g = torch.Generator().manual_seed(b * 100 + S * 10 + Hq + 7)
+    x = torch.randn(b, S, K, generator=g).to(dtype).to(dev)
+    w = (torch.randn((Hq + 2 * Hkv) * D, K, generator=g) * 0.05).to(dtype).to(dev)
+    qw = (1 + 0.1 * torch.randn(D, generator=g)).to(dtype).to(dev)
+    kw = (1 + 0.1 * torch.randn(D, generator=g)).to(dtype).to(dev)
+    cos, sin, _ = _rope_tables(S, D, dtype=dtype)
+    cos, sin = cos.to(dev), sin.to(dev)
+    qkv = linear_rows(x, w)
+    q = qkv[..., : Hq * D].view(b, S, Hq, D)
+    k = qkv[..., Hq * D: (Hq + Hkv) * D].view(b, S, Hkv, D)
+    v = qkv[..., (Hq + Hkv) * D:].view(b, S, Hkv, D)
+    q0, k0, v0 = ksa_amd.pre_attention(q, k, v, qw, kw, cos, sin, eps=1e-6)
+    cap = 64
+    kc = torch.full((b, Hkv, cap, D), 7.0, dtype=dtype, device=dev)
+    vc = torch.full((b, Hkv, cap, D), -3.0, dtype=dtype, device=dev)
+    # token 0 at a per-sequence cursor, the others in a run of rows elsewhere (also per sequence)
+    table = torch.empty(b, S, dtype=torch.int32)
+    for i in range(b):
+        table[i, 0] = 40 + (i * 5) % 20
+        table[i, 1:] = torch.arange(S - 1) + (i % 3) * 10
+    table = table.to(dev)
+    slots = dict(k_out=kc[:, :, :S].transpose(1, 2), v_out=vc[:, :, :S].transpose(1, 2), kv_out_row=table)
+    if from_partials:
+        d = linear_rows(x, w, defer=True)
+        if not isinstance(d, SplitKPartials):
+            pytest.skip("this shape is not split over K")
+        q1, _, _ = pre_attention_partials(d, Hq, Hkv, D, qw, kw, cos, sin, eps=1e-6, **slots)
+    else:
+        q1, _, _ = ksa_amd.pre_attention(q, k, v, qw, kw, cos, sin, eps=1e-6, **slots)
+    torch.cuda.synchronize()
+    assert torch.equal(q0, q1)
+    touched = torch.zeros(b, cap, dtype=torch.bool)
+    for i in range(b):
+        for t in range(S):
+            r = int(table[i, t])
+            touched[i, r] = True
+            assert torch.equal(kc[i, :, r], k0[i, t]) and torch.equal(vc[i, :, r], v0[i, t])
+    untouched = ~touched.to(dev)
+    assert (kc.transpose(1, 2)[untouched] == 7.0).all() and (vc.transpose(1, 2)[untouched] == -3.0).all()
