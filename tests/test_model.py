@@ -228,6 +228,28 @@ def test_gpu_module_matches_cpu_module(S, D, indep, mix):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("batch,S", [(20, 2), (40, 1), (64, 1)])
+def test_gpu_module_more_than_16_rows(batch, S):
+    """A batch above 16: the steps inside a chunk (`batch` rows) and the chunk-boundary steps (batch x (1 + S)
+    rows, up to 128) run their projections on the wide form of the few-rows GEMMs, with the K-split partial
+    sums handed to the norms and the pre-attention step, and the MLP as two launches.  Same check and
+    tolerance as `test_gpu_module_matches_cpu_module`; then the same steps replayed from HIP graphs against
+    the eager ones."""
+    from ksa_amd.model import HipOps
+    cfg = tiny_config(summary_token_num=S, head_dim=64, hidden_size=128, intermediate_size=256)
+    rel, agree = _gpu_vs_cpu(cfg, batch=batch, n_prompt=21, n_new=20, seed=5, tol_rel=1.5e-2)
+    print(f"max logit error {rel:.3e} of the logit scale, arg-max agreement {agree:.2f}")
+    _, w = cpu_model(cfg, 5)
+    gpu = KsaQwen3ForCausalLM(cfg, convert_weights(w, "cuda", torch.bfloat16), HipOps())
+    gpu.BOUNDARY_GRAPH_AFTER = 0
+    ids = torch.randint(0, cfg.vocab_size, (batch, 21), generator=torch.Generator().manual_seed(6))
+    out_e, log_e = gpu.generate(ids, 40, return_logits=True)
+    out_g, log_g = gpu.generate(ids, 40, forced=out_e[:, 21:], return_logits=True, use_graph=True)
+    scale = log_e.abs().max().item()
+    assert (log_g - log_e).abs().max().item() <= 1e-2 * scale
+
+
+@pytest.mark.gpu
 def test_gpu_module_kernel_shape():
     """The real attention shape (C=128, S=8, 8/2 heads, D=128, windows 1 | unbounded | 1):
     prefill of 300 tokens, 120 decode steps (one boundary), batch 2."""
