@@ -217,26 +217,18 @@ __global__ __launch_bounds__(64 * kWideWaves) void ksa_gemm_rows_wide_kernel(con
         }
     };
     if (c_begin < c_end) {  // (uniform; an empty slice does not exist in a grid made by wide_plan)
-        // The workgroups of a launch walk their chunks in rotated orders: rows of w are K elements apart,
-        // and with every workgroup at the same offset inside its rows at the same time the requests of the
-        // whole grid meet in a few memory channels.
-        const int nch = c_end - c_begin;
-        int c = c_begin + (int)(blockIdx.x % (unsigned)nch);
-        auto next = [&](int cc) { return cc + 1 < c_end ? cc + 1 : c_begin; };
-        x_request(c);
+        x_request(c_begin);
 #pragma unroll
-        for (int u = 0; u < kChunkSteps; ++u) w_request(c, u);
-        x_store(c);
+        for (int u = 0; u < kChunkSteps; ++u) w_request(c_begin, u);
+        x_store(c_begin);
         __syncthreads();
-        for (int k = 0; k + 1 < nch; ++k) {
-            const int cn = next(c);
-            chunk(std::true_type{}, cn);
+        for (int c = c_begin; c + 1 < c_end; ++c) {
+            chunk(std::true_type{}, c + 1);
             __syncthreads();  // every wave is done with this chunk of x
-            x_store(cn);
+            x_store(c + 1);
             __syncthreads();
-            c = cn;
         }
-        chunk(std::false_type{}, c);
+        chunk(std::false_type{}, c_end);
     }
     // C layout of a 16x16 tile: lane holds row (of x) lane % 16 of the block, columns n0 + 4 * (lane / 16) + i
     const int n = n0 + 4 * kq;
