@@ -283,6 +283,19 @@ int ksa_silu_mul_partials(const float* partials, int ksplit, void* out, int rows
  * KSA_ERR_INVALID.  With ksplit > 1 out may be NULL: the partial sums (fp32 [ksplit][R][N], R = M
  * rounded up to a multiple of 16) are then left in the workspace for a consumer that adds them itself
  * (ksa_add_rmsnorm_partials, ksa_silu_mul_partials, ksa_pre_attention_partials). */
+/* The streaming layout of a weight matrix.  The few-rows kernels read a weight fragment of 16 rows x 32
+ * elements of K per wave instruction - in a row-major w [N, K] that is 64 bytes of each of 16 rows K elements
+ * apart.  ksa_tile_weights writes the same matrix as [ceil(N / 16)][K / 32][16][32] (rows past N: zeros;
+ * ksa_tile_weights_bytes(N, K) bytes, 16-byte aligned), in which a fragment is 1 KB in one piece and a wave's
+ * share of the matrix one sequential run; a caller that has the memory keeps this second copy of the
+ * projection weights for its decode steps (measured on the 4B-shape projections: q|k|v -7 %, down -15 %,
+ * gate|up -10 % of the kernel time).  Such a matrix is passed as `w` with KSA_W_TILED in place of its row
+ * stride to ksa_gemm_rows, ksa_gemm_rows_gate_up_silu (I a multiple of 16), ksa_mlp_rows and
+ * ksa_add_rmsnorm_mlp_rows; results are bit-identical to the row-major call.  K a multiple of 32. */
+#define KSA_W_TILED (-1LL)
+size_t ksa_tile_weights_bytes(int N, int K);
+int ksa_tile_weights(const void* w, void* out, int N, int K, long long w_row_stride, void* stream);
+
 int ksa_gemm_rows_auto_splits(int N, int K);
 size_t ksa_gemm_rows_workspace_bytes(int N, int ksplit);
 int ksa_gemm_rows_splits(int M, int N, int K);

@@ -49,6 +49,8 @@ _SIGNATURES = {
     "ksa_silu_mul_partials": (_int, [_vp, _int, _vp, _int, _int, ctypes.c_longlong, _int, _vp]),
     "ksa_gemm_rows_auto_splits": (_int, [_int, _int]),
     "ksa_gemm_rows_workspace_bytes": (ctypes.c_size_t, [_int, _int]),
+    "ksa_tile_weights_bytes": (ctypes.c_size_t, [_int, _int]),
+    "ksa_tile_weights": (_int, [_vp, _vp, _int, _int, ctypes.c_longlong, _vp]),
     "ksa_gemm_rows_splits": (_int, [_int, _int, _int]),
     "ksa_gemm_rows_partials_bytes": (ctypes.c_size_t, [_int, _int, _int]),
     "ksa_gemm_rows": (_int, [_vp] * 3 + [_int] * 3 + [ctypes.c_longlong] * 3 + [_int, _int, _vp, ctypes.c_size_t, _vp]),

@@ -16,6 +16,9 @@ enum {
 
 enum { KSA_DTYPE_BF16 = 0, KSA_DTYPE_F16 = 1 };
 
+// value of a weight matrix's row stride that names the streaming layout instead (include/ksa_hip.h, KSA_W_TILED)
+constexpr long long kWTiled = -1;
+
 // most rows of x that the few-rows GEMM (ksa_gemm_rows) and the consumers of its K-split partial sums take
 constexpr int kMaxPartialRows = 128;
 

@@ -49,8 +49,7 @@ __global__ __launch_bounds__(256) void ksa_gemm_rows_kernel(const GemmParams p) 
     const int s_begin = blockIdx.y * per_split;
     const int s_end = min(steps, s_begin + per_split);
 
-    const int nrow = min(n0 + r, p.N - 1);
-    const uint16_t* wp = p.w + (int64_t)nrow * p.ws + 8 * kq;
+    const KsaWeightLane wl = ksa_weight_lane(p.w, p.ws, p.K, n0, r, kq, p.N);
     // rows of x beyond M repeat the last one: their columns of the product are never stored
     const int xrow = min(r, p.M - 1);
 
@@ -60,7 +59,7 @@ __global__ __launch_bounds__(256) void ksa_gemm_rows_kernel(const GemmParams p) 
         const int nst = min(kChunkSteps, s_end - c0);
         u32x4 a[kChunkSteps];
 #pragma unroll
-        for (int u = 0; u < kChunkSteps; ++u) a[u] = *reinterpret_cast<const u32x4*>(wp + 32 * min(c0 + u, s_end - 1));
+        for (int u = 0; u < kChunkSteps; ++u) a[u] = *reinterpret_cast<const u32x4*>(wl.p + wl.step * min(c0 + u, s_end - 1));
         // x[0:M][32 c0 .. 32 (c0 + nst)) -> LDS, 16 bytes per thread and pass
         for (int e = threadIdx.x; e < p.M * (kChunkK / 8); e += 256) {
             const int m = e / (kChunkK / 8), j = e % (kChunkK / 8);
@@ -137,20 +136,19 @@ __global__ __launch_bounds__(64 * kWideWaves) void ksa_gemm_rows_wide_kernel(con
     const int r = lane & 15;   // row of W inside the wave's tile (A operand) / row of x inside a block (B operand)
     const int kq = lane >> 4;  // which 8 of the 32 K elements of a step
     int n0;                    // first output column of this wave (kPair: of the gate / up half)
-    int64_t wrow;              // this lane's row of w
+    KsaWeightLane wl;          // this lane's piece of the wave's weight fragments
     if constexpr (kPair) {
         const int half = wave / (nw / 2);
         n0 = (blockIdx.x * (nw / 2) + wave % (nw / 2)) * 16;
-        wrow = (int64_t)half * p.N + min(n0 + r, p.N - 1);
+        wl = ksa_weight_lane(p.w, p.ws, p.K, (int64_t)half * p.N + n0, r, kq, (int64_t)(half + 1) * p.N);
     } else {
         n0 = (blockIdx.x * nw + wave) * 16;
-        wrow = min(n0 + r, p.N - 1);
+        wl = ksa_weight_lane(p.w, p.ws, p.K, n0, r, kq, p.N);
     }
     const int steps = p.K / 32;
     const int chunks = (steps + kChunkSteps - 1) / kChunkSteps;
     const int c_begin = blockIdx.y * p.chunks_per_split;
     const int c_end = min(chunks, c_begin + p.chunks_per_split);
-    const uint16_t* wp = p.w + wrow * p.ws + 8 * kq;
 
     f32x4 acc[MB];
 #pragma unroll
@@ -190,7 +188,7 @@ __global__ __launch_bounds__(64 * kWideWaves) void ksa_gemm_rows_wide_kernel(con
     };
     u32x4 a[kChunkSteps];
     auto w_request = [&](int c, int u) {
-        a[u] = *reinterpret_cast<const u32x4*>(wp + 32 * min(c * kChunkSteps + u, steps - 1));
+        a[u] = *reinterpret_cast<const u32x4*>(wl.p + wl.step * min(c * kChunkSteps + u, steps - 1));
     };
     // the products of one chunk; kMore: there is a next chunk, whose x and weights are requested on the way
     // (two copies of the loop body rather than a condition inside it: with branches between the MFMAs the
@@ -385,7 +383,7 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) vo
     const int steps = p.K / 32;
     const int chunks = (steps + kChunkSteps - 1) / kChunkSteps;
     const int rowb = (p.K + 8) * 2;
-    const uint16_t* wp = p.w + ((int64_t)half * p.I + min(n0 + r, p.I - 1)) * p.ws + 8 * kq;
+    const KsaWeightLane wl = ksa_weight_lane(p.w, p.ws, p.K, (int64_t)half * p.I + n0, r, kq, (int64_t)(half + 1) * p.I);
     const int xrow = min(r, p.M - 1);
 
     // eight K steps of weights in flight per wave (32 registers): with at most 64 registers a SIMD
@@ -395,7 +393,7 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) vo
     u32x4 a[kB];
     auto load_steps = [&](int s0) {
 #pragma unroll
-        for (int u = 0; u < kB; ++u) a[u] = *reinterpret_cast<const u32x4*>(wp + 32 * min(s0 + u, steps - 1));
+        for (int u = 0; u < kB; ++u) a[u] = *reinterpret_cast<const u32x4*>(wl.p + wl.step * min(s0 + u, steps - 1));
     };
     load_steps(slice * kChunkSteps);  // in flight while x is staged (every slice has a first chunk: S <= chunks)
     const int per_row = p.K / 8;
@@ -489,7 +487,7 @@ extern "C" int ksa_gemm_rows(const void* x, const void* w, void* out, int M, int
     if (M <= 0 || M > kMaxPartialRows || N <= 0 || K <= 0 || K % 32 != 0 || ksplit < 1 || ksplit > 64) return KSA_ERR_INVALID;
     if (dtype != KSA_DTYPE_BF16 && dtype != KSA_DTYPE_F16) return KSA_ERR_UNSUPPORTED;
     if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w)) & 15) return KSA_ERR_ALIGN;
-    if (x_row_stride % 8 || w_row_stride % 8) return KSA_ERR_ALIGN;
+    if (x_row_stride % 8 || (w_row_stride != kWTiled && w_row_stride % 8)) return KSA_ERR_ALIGN;
     if (M > 16) {
         const WidePlan pl = wide_plan(K, ksplit);
         if (pl.ksplit != ksplit) return KSA_ERR_INVALID;  // not a split count of ksa_gemm_rows_splits: an empty slice
@@ -537,7 +535,8 @@ extern "C" int ksa_gemm_rows_gate_up_silu(const void* x, const void* w, void* ou
     if (M <= 0 || M > kMaxPartialRows || I <= 0 || K <= 0 || K % 32 != 0) return KSA_ERR_INVALID;
     if (dtype != KSA_DTYPE_BF16 && dtype != KSA_DTYPE_F16) return KSA_ERR_UNSUPPORTED;
     if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w)) & 15) return KSA_ERR_ALIGN;
-    if (x_row_stride % 8 || w_row_stride % 8) return KSA_ERR_ALIGN;
+    if (x_row_stride % 8 || (w_row_stride != kWTiled && w_row_stride % 8)) return KSA_ERR_ALIGN;
+    if (w_row_stride == kWTiled && I % 16 != 0) return KSA_ERR_UNSUPPORTED;  // gate and up rows must start tiles of their own
     if (M > 16) {  // chunks of x through LDS, gate and up waves of a workgroup meet behind the walk
         WideParams wp{};
         wp.x = (const uint16_t*)x, wp.w = (const uint16_t*)w, wp.out = (uint16_t*)out;
@@ -565,5 +564,38 @@ extern "C" int ksa_gemm_rows_gate_up_silu(const void* x, const void* w, void* ou
         if (e != hipSuccess) return KSA_ERR_LAUNCH;
     }
     hipLaunchKernelGGL(kern, grid, block, lds, (hipStream_t)stream, p);
+    return ksa_check_launch();
+}
+
+// ---- the streaming layout of a weight matrix ----
+namespace {
+// out [ceil(N / 16)][K / 32][16][32] <- w [N, K] (rows past N: zeros); 16 bytes per thread
+__global__ __launch_bounds__(256) void ksa_tile_weights_kernel(const uint16_t* w, uint16_t* out, int N, int K, int64_t ws) {
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;  // 16-byte piece of the output
+    const int steps = K / 32;
+    const int64_t total = (int64_t)((N + 15) / 16) * steps * 64;
+    if (e >= total) return;
+    const int q = (int)(e & 3), r = (int)((e >> 2) & 15);
+    const int64_t frag = e >> 6;
+    const int s = (int)(frag % steps);
+    const int64_t row = (frag / steps) * 16 + r;
+    u32x4 v = {0u, 0u, 0u, 0u};
+    if (row < N) v = *reinterpret_cast<const u32x4*>(w + row * ws + 32 * s + 8 * q);
+    *reinterpret_cast<u32x4*>(out + 8 * e) = v;
+}
+}  // namespace
+
+extern "C" size_t ksa_tile_weights_bytes(int N, int K) {
+    return N > 0 && K > 0 ? (size_t)((N + 15) / 16 * 16) * (size_t)K * 2 : 0;
+}
+
+extern "C" int ksa_tile_weights(const void* w, void* out, int N, int K, long long w_row_stride, void* stream) {
+    if (!w || !out) return KSA_ERR_NULL;
+    if (N <= 0 || K <= 0 || K % 32 != 0) return KSA_ERR_INVALID;
+    if ((reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(out)) & 15) return KSA_ERR_ALIGN;
+    if (w_row_stride % 8) return KSA_ERR_ALIGN;
+    const int64_t total = (int64_t)((N + 15) / 16) * (K / 32) * 64;
+    hipLaunchKernelGGL(ksa_tile_weights_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       (const uint16_t*)w, (uint16_t*)out, N, K, (int64_t)w_row_stride);
     return ksa_check_launch();
 }

@@ -183,13 +183,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
         const int slice = wave - half * kSlices;
         const int sl_steps = p.H / 32 / kSlices;  // K steps of a slice (H is a multiple of 128)
         const int rowb = (p.H + 8) * 2;
-        const uint16_t* wp = p.w_gu + ((int64_t)half * p.I + min(kTileCols * u + (r & (kTileCols - 1)), p.I - 1)) * p.wgu_rs +
-                             32 * (slice * sl_steps) + 8 * kq;
+        static_assert(kTileCols == 16, "a workgroup's columns are one tile of the streaming weight layout");
+        KsaWeightLane wl = ksa_weight_lane(p.w_gu, p.wgu_rs, p.H, (int64_t)half * p.I + kTileCols * u, r, kq,
+                                           (int64_t)(half + 1) * p.I);
+        wl.p += (int64_t)wl.step * (slice * sl_steps);
         auto load_steps = [&](int s0) {  // (steps beyond the slice repeat its last one and are not multiplied)
             if (r < kTileCols) {
 #pragma unroll
                 for (int k = 0; k < kB; ++k)
-                    a[k] = *reinterpret_cast<const u32x4*>(wp + 32 * min(s0 + k, sl_steps - 1));
+                    a[k] = *reinterpret_cast<const u32x4*>(wl.p + wl.step * min(s0 + k, sl_steps - 1));
             }
         };
         load_steps(0);  // in flight while x is waited for and staged
@@ -283,13 +285,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
     const int s0c = kc * kChunkSteps;
     const int nst = min(kChunkSteps, stepsI - s0c);
     const bool live = ct < CT;
-    const uint16_t* wp = p.w_dn + (int64_t)(16 * min(ct, CT - 1) + r) * p.wdn_rs + 32 * s0c + 8 * kq;  // (dead behind the requests)
+    KsaWeightLane wl = ksa_weight_lane(p.w_dn, p.wdn_rs, p.I, 16 * min(ct, CT - 1), r, kq, p.H);  // (dead behind the requests)
+    wl.p += (int64_t)wl.step * s0c;
     // all 16 steps of the chunk are requested at once (steps beyond its end repeat the last one and
     // are not multiplied): nothing but the activation is waited for once the chunk's tiles are there
     u32x4 ad[kChunkSteps];
     if (live) {  // on their way while the activation is waited for
 #pragma unroll
-        for (int k = 0; k < kChunkSteps; ++k) ad[k] = *reinterpret_cast<const u32x4*>(wp + 32 * min(k, nst - 1));
+        for (int k = 0; k < kChunkSteps; ++k) ad[k] = *reinterpret_cast<const u32x4*>(wl.p + wl.step * min(k, nst - 1));
     }
     unsigned long long launch = 0;  // (thread 0 only) launches before this one
     if (tid == 0) {
@@ -398,7 +401,8 @@ int mlp_rows_launch(const void* x, long long x_row_stride, const float* o_partia
     if (workspace_bytes < ksa_mlp_rows_workspace_bytes(H, I)) return KSA_ERR_WORKSPACE;
     auto bad = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) != 0; };
     if (bad(w_gate_up) || bad(w_down) || bad(down_partials) || bad(workspace)) return KSA_ERR_ALIGN;
-    if (w_gate_up_row_stride % 8 || w_down_row_stride % 8) return KSA_ERR_ALIGN;
+    if ((w_gate_up_row_stride != kWTiled && w_gate_up_row_stride % 8) || (w_down_row_stride != kWTiled && w_down_row_stride % 8))
+        return KSA_ERR_ALIGN;
     const size_t lds = mlp_lds_bytes(M, H);
     if (lds > 160 * 1024) return KSA_ERR_UNSUPPORTED;
     auto kern = dtype == KSA_DTYPE_BF16 ? ksa_mlp_rows_kernel<KsaBf16> : ksa_mlp_rows_kernel<KsaF16>;

@@ -3,6 +3,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include "ksa_api_internal.h"
 #include "ksa_cvt.h"
 
 
@@ -24,3 +25,27 @@ __device__ __forceinline__ f32x4 mfma16<KsaF16>(u32x4 a, u32x4 b, f32x4 c) {
 constexpr int kChunkSteps = 16;                 // K steps (of 32) per staged chunk of x
 constexpr int kChunkK = 32 * kChunkSteps;       // 512 elements of K
 constexpr int kRowB = (kChunkK + 8) * 2;        // padded LDS row of x in bytes (conflict-free b128 reads)
+
+// Where a lane finds its 16 bytes of a weight fragment (16 rows of w x 32 elements of K, the A operand of
+// one MFMA; lane = (row r of the 16, quarter kq of the 32)).  Row-major w [N, K]: row n starts n * rs
+// elements in, the fragment of K step s lies 32 s elements further - 64 bytes of each of 16 rows that are
+// K elements apart.  Streaming layout (rs == kWTiled, made by ksa_tile_weights): the 1 KB of a fragment is
+// contiguous and the K / 32 fragments of 16 rows follow one another, [ceil(N / 16)][K / 32][16][32], so a
+// wave reads its rows' share of the matrix as one sequential run (rows past N are zeros).
+struct KsaWeightLane {
+    const uint16_t* p;  // this lane's piece of K step 0
+    int step;           // elements from one K step to the next
+};
+__device__ __forceinline__ KsaWeightLane ksa_weight_lane(const uint16_t* w, int64_t rs, int K, int64_t row0, int r,
+                                                         int kq, int64_t nrows) {
+    KsaWeightLane l;
+    if (rs == kWTiled) {
+        l.p = w + (row0 / 16) * (int64_t)(K / 32) * 512 + r * 32 + 8 * kq;
+        l.step = 512;
+    } else {
+        const int64_t row = row0 + r < nrows ? row0 + r : nrows - 1;
+        l.p = w + row * rs + 8 * kq;
+        l.step = 32;
+    }
+    return l;
+}

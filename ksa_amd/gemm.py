@@ -17,6 +17,39 @@ MAX_ROWS = 128       # rows of x the GEMM kernels take
 MLP_MAX_ROWS = 16    # rows the one-launch MLP takes (x whole in LDS)
 
 
+W_TILED = -1   # row stride that names the streaming layout (include/ksa_hip.h, KSA_W_TILED)
+
+
+class TiledWeight:
+    """A weight matrix [N, K] in the streaming layout of the few-rows kernels, [ceil(N / 16)][K / 32][16][32]
+    (`ksa_tile_weights`): what a wave reads of it is one sequential run instead of 64-byte pieces of rows K
+    elements apart.  A second copy of the matrix for the decode steps; `linear_rows`, `gate_up_silu_rows`,
+    `mlp_rows` and `add_rmsnorm_mlp_rows` take it in place of the tensor, with bit-identical results."""
+
+    def __init__(self, weight: torch.Tensor):
+        assert weight.is_cuda and weight.dtype in _DT and weight.dim() == 2 and weight.stride(1) == 1
+        N, K = weight.shape
+        assert K % 32 == 0, "K must be a multiple of 32"
+        L = _lib.lib()
+        self.shape, self.dtype, self.device = (N, K), weight.dtype, weight.device
+        self.data = torch.empty(L.ksa_tile_weights_bytes(N, K) // 2, dtype=weight.dtype, device=weight.device)
+        with torch.cuda.device(weight.device):
+            rc = L.ksa_tile_weights(weight.data_ptr(), self.data.data_ptr(), N, K, weight.stride(0),
+                                    _lib.stream_ptr(weight.device))
+        _lib.check(rc, "ksa_tile_weights")
+
+    def stride(self, dim):
+        return W_TILED if dim == 0 else 1
+
+    def data_ptr(self):
+        return self.data.data_ptr()
+
+
+def _weight_ok(weight, N, K, dtype):
+    """Shape / dtype / layout check of a weight operand (a tensor with contiguous rows, or a `TiledWeight`)."""
+    return tuple(weight.shape) == (N, K) and weight.dtype == dtype and weight.stride(1) == 1
+
+
 class SplitKPartials:
     """Output of `linear_rows(..., defer=True)` when K was split over workgroups: the fp32 partial
     sums [ksplit, rows rounded up to whole 16-row blocks, N] as the kernel left them, for a consumer that adds them itself
@@ -36,7 +69,7 @@ def linear_rows(x: torch.Tensor, weight: torch.Tensor, defer: bool = False):
     assert x.is_cuda and x.dtype in _DT and weight.dtype == x.dtype, "bf16/fp16 GPU tensors"
     K = x.shape[-1]
     N = weight.shape[0]
-    assert weight.shape == (N, K) and weight.stride(1) == 1
+    assert _weight_ok(weight, N, K, x.dtype)
     x2 = x.reshape(-1, K)
     if x2.stride(1) != 1:
         x2 = x2.contiguous()
@@ -69,7 +102,7 @@ def gate_up_silu_rows(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     assert x.is_cuda and x.dtype in _DT and weight.dtype == x.dtype, "bf16/fp16 GPU tensors"
     K = x.shape[-1]
     I = weight.shape[0] // 2
-    assert weight.shape == (2 * I, K) and weight.stride(1) == 1
+    assert _weight_ok(weight, 2 * I, K, x.dtype)
     x2 = x.reshape(-1, K)
     if x2.stride(1) != 1:
         x2 = x2.contiguous()
@@ -125,8 +158,7 @@ def mlp_rows(x: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor, ws:
     I = w_gate_up.shape[0] // 2
     dt = x.dtype
     assert x.is_cuda and dt in _DT
-    assert w_gate_up.shape == (2 * I, H) and w_down.shape == (H, I) and w_gate_up.dtype == dt and w_down.dtype == dt
-    assert w_gate_up.stride(1) == 1 and w_down.stride(1) == 1 and ws.H == H and ws.I == I
+    assert _weight_ok(w_gate_up, 2 * I, H, dt) and _weight_ok(w_down, H, I, dt) and ws.H == H and ws.I == I
     x2 = x.reshape(-1, H)
     if x2.stride(1) != 1:
         x2 = x2.contiguous()
@@ -151,8 +183,7 @@ def add_rmsnorm_mlp_rows(o_partials: SplitKPartials, residual: torch.Tensor, nor
     I = w_gate_up.shape[0] // 2
     M = o_partials.rows
     dt = o_partials.dtype
-    assert w_gate_up.shape == (2 * I, H) and w_down.shape == (H, I) and w_gate_up.dtype == dt and w_down.dtype == dt
-    assert w_gate_up.stride(1) == 1 and w_down.stride(1) == 1 and ws.H == H and ws.I == I and H <= 4096
+    assert _weight_ok(w_gate_up, 2 * I, H, dt) and _weight_ok(w_down, H, I, dt) and ws.H == H and ws.I == I and H <= 4096
     r2 = residual.reshape(-1, H)
     if r2.stride(1) != 1:
         r2 = r2.contiguous()

@@ -151,6 +151,23 @@ class HipOps:
         self._mlp_ws = {}   # (device, H, I) -> MlpRowsWorkspace, see `mlp_rows`
         # False: the MLP of a decode step runs as separate launches (set after a one-launch MLP timed out)
         self.mlp_one_launch = True
+        # True: the few-rows kernels of the decode steps read a second copy of every projection matrix in
+        # their streaming layout (`gemm.TiledWeight`: + the size of those matrices in device memory, made the
+        # first time a matrix is used at a decode step; q|k|v -7 %, down -15 %, gate|up -10 % of the kernel time)
+        self.tile_weights = True
+        self._tiled = {}    # (address, shape, row stride) -> (the matrix, its TiledWeight)
+
+    def _streaming(self, weight, multiple=16):
+        """`weight` in the streaming layout (kept with the matrix it was made from, so that the key stays
+        unique for as long as the copy exists); the matrix itself where that layout does not apply."""
+        if not self.tile_weights or not torch.is_tensor(weight) or weight.dim() != 2 or weight.stride(1) != 1 \
+                or weight.shape[1] % 32 or weight.shape[0] % multiple or weight.stride(0) % 8:
+            return weight
+        key = (weight.data_ptr(), tuple(weight.shape), weight.stride(0))
+        hit = self._tiled.get(key)
+        if hit is None:
+            hit = self._tiled[key] = (weight, self._gemm.TiledWeight(weight))
+        return hit[1]
 
     def decode(self, q, kbuf, vbuf, start, end, scale):
         return self._decode(q, kbuf, vbuf, start, end, scale=scale)
@@ -177,7 +194,8 @@ class HipOps:
         H, I = x.shape[-1], w_down.shape[1]
         if not self.mlp_one_launch or not self._gemm.mlp_rows_supported(rows, H, I):
             return None
-        return self._gemm.mlp_rows(x, w_gate_up, w_down, self.prepare_mlp_rows(H, I, x.device))
+        return self._gemm.mlp_rows(x, self._streaming(w_gate_up, 32), self._streaming(w_down),
+                                   self.prepare_mlp_rows(H, I, x.device))
 
     def add_norm_mlp_rows(self, o_partials, residual, norm_weight, eps, w_gate_up, w_down):
         """(residual + o_proj output, down(SiLU(gate(h)) * up(h)) for h = norm of that sum) in one launch,
@@ -188,8 +206,8 @@ class HipOps:
         H, I = residual.shape[-1], w_down.shape[1]
         if not self._gemm.mlp_rows_supported(o_partials.rows, H, I) or H > 4096:
             return None
-        return self._gemm.add_rmsnorm_mlp_rows(o_partials, residual, norm_weight, eps, w_gate_up, w_down,
-                                               self.prepare_mlp_rows(H, I, residual.device))
+        return self._gemm.add_rmsnorm_mlp_rows(o_partials, residual, norm_weight, eps, self._streaming(w_gate_up, 32),
+                                               self._streaming(w_down), self.prepare_mlp_rows(H, I, residual.device))
 
     def mlp_rows_failed(self):
         """True if a `mlp_rows` launch gave up waiting since the last call (waits for the device; every
@@ -212,9 +230,9 @@ class HipOps:
         rows = x.numel() // x.shape[-1]
         k = x.shape[-1]
         if rows <= self._max_rows and k % 32 == 0 and (rows > 16 or rows * (k + 8) * 2 <= 160 * 1024):
-            return self._gate_up_silu_rows(x, weight)
+            return self._gate_up_silu_rows(x, self._streaming(weight, 32))
         if rows <= self._max_rows:
-            return self.silu_mul(self._linear_rows(x, weight, defer=True))
+            return self.silu_mul(self._linear_rows(x, self._streaming(weight), defer=True))
         return self.silu_mul(F.linear(x, weight))
 
     def linear(self, x, weight, defer=False):
@@ -223,7 +241,7 @@ class HipOps:
         product split over K may come back as its partial sums (one launch less)."""
         rows = x.numel() // x.shape[-1]
         if rows <= self._max_rows and x.shape[-1] % 32 == 0:
-            return self._linear_rows(x, weight, defer=defer)
+            return self._linear_rows(x, self._streaming(weight), defer=defer)
         return F.linear(x, weight)
 
 

@@ -297,3 +297,60 @@ def test_gpu_mlp_rows_bounded_wait_gives_up_and_recovers():
     assert not ws.failed()
     assert torch.equal(got.workspace.view(torch.float32).view(got.ksplit, 16, H)[:, :M],
                        want.workspace.view(torch.float32).view(want.ksplit, 16, H)[:, :M])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_gpu_streaming_weight_layout(dtype):
+    """`TiledWeight` (`ksa_tile_weights`): [ceil(N / 16)][K / 32][16][32] with zero rows past N, from a
+    matrix and from a row slice of a larger one; and every few-rows kernel gives bit for bit the result
+    of the row-major call on it (same products in the same order, only the addresses differ)."""
+    from ksa_amd.gemm import (MlpRowsWorkspace, TiledWeight, add_rmsnorm_mlp_rows, gate_up_silu_rows, linear_rows,
+                              mlp_rows)
+    dev = torch.device("cuda")
+    g = torch.Generator().manual_seed(11)
+
+    def sums(d):  # the rows of the partial sums that exist (a slice holds whole 16-row blocks)
+        return d.workspace.view(torch.float32).view(d.ksplit, -1, d.shape[-1])[:, :d.rows]
+    for N, K in ((40, 96), (2560, 4096), (1000, 640)):
+        big = (torch.randn(N + 8, K + 64, generator=g) * 0.05).to(dtype).to(dev)
+        w = big[8:, :K]                                   # rows 8.., a row stride above K
+        t = TiledWeight(w)
+        Np = (N + 15) // 16 * 16
+        ref = torch.zeros(Np, K, dtype=dtype, device=dev)
+        ref[:N] = w
+        ref = ref.view(Np // 16, 16, K // 32, 32).permute(0, 2, 1, 3).contiguous().view(-1)
+        assert torch.equal(t.data, ref)
+        for M in (1, 8, 16, 17, 72, 128):
+            x = torch.randn(M, K, generator=g).to(dtype).to(dev)
+            assert torch.equal(linear_rows(x, t), linear_rows(x, w)), (N, K, M)
+    # deferred partial sums as well
+    w = (torch.randn(2560, 4096, generator=g) * 0.05).to(dtype).to(dev)
+    t = TiledWeight(w)
+    for M in (8, 72):
+        x = torch.randn(M, 4096, generator=g).to(dtype).to(dev)
+        a, b = linear_rows(x, t, defer=True), linear_rows(x, w, defer=True)
+        assert a.ksplit == b.ksplit and torch.equal(sums(a), sums(b))
+    # gate | up with the activation, the one-launch MLP, and the MLP with the norm in front
+    H, I = 1024, 768
+    w_gu = (torch.randn(2 * I, H, generator=g) * 0.04).to(dtype).to(dev)
+    w_dn = (torch.randn(H, I, generator=g) * 0.03).to(dtype).to(dev)
+    t_gu, t_dn = TiledWeight(w_gu), TiledWeight(w_dn)
+    for M in (3, 16, 40, 128):
+        x = torch.randn(1, M, H, generator=g).to(dtype).to(dev)
+        assert torch.equal(gate_up_silu_rows(x, t_gu), gate_up_silu_rows(x, w_gu)), M
+    ws = MlpRowsWorkspace(H, I, dev)
+    for M in (1, 8, 16):
+        x = torch.randn(1, M, H, generator=g).to(dtype).to(dev)
+        a, b = mlp_rows(x, t_gu, t_dn, ws), mlp_rows(x, w_gu, w_dn, ws)
+        assert torch.equal(sums(a), sums(b)), M
+        w_o = (torch.randn(H, 512, generator=g) * 0.05).to(dtype).to(dev)
+        attn = torch.randn(1, M, 512, generator=g).to(dtype).to(dev)
+        res = torch.randn(1, M, H, generator=g).to(dtype).to(dev)
+        nw = (1 + 0.1 * torch.randn(H, generator=g)).to(dtype).to(dev)
+        o = linear_rows(attn, TiledWeight(w_o), defer=True)
+        if isinstance(o, type(a)):
+            s1, d1 = add_rmsnorm_mlp_rows(o, res, nw, 1e-6, t_gu, t_dn, ws)
+            s0, d0 = add_rmsnorm_mlp_rows(o, res, nw, 1e-6, w_gu, w_dn, ws)
+            assert torch.equal(s0, s1) and torch.equal(sums(d0), sums(d1)), M
+    assert not ws.failed()
