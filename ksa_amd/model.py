@@ -310,11 +310,11 @@ class KsaQwen3ForCausalLM:
     greedy loop.  All sequences of a batch have the same length."""
 
     # `decode_step_graph` runs this many chunk-boundary steps of a cache eagerly before it records
-    # them: a replayed boundary step saves about 4 ms against an eager one (7.4 against 11.3 ms at the
-    # 4B shape, batch 8), its recording costs about 24 ms of host time (an eager run outside the
-    # capture first, then the capture), i.e. six boundaries' worth: so a short generation never pays
-    # for a recording it does not use, and a long one pays at most twice the best possible.
-    BOUNDARY_GRAPH_AFTER = 6
+    # them: a replayed boundary step saves about 1 ms against an eager one (6.2 against 7.2 ms at the
+    # 4B shape, batch 8), its recording costs about 17 ms more than an eager step (an eager run outside
+    # the capture first, then the capture), i.e. sixteen boundaries' worth: so a short generation never
+    # pays for a recording it does not use, and a long one pays at most twice the best possible.
+    BOUNDARY_GRAPH_AFTER = 16
 
     def __init__(self, config: KsaQwen3Config, weights: dict, ops=None):
         self.config = config

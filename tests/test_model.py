@@ -342,15 +342,15 @@ def test_gpu_graph_decode_survives_buffer_growth():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("S,indep,mix,after", [(1, False, 1.0, 0), (2, True, 0.35, 0), (2, False, 1.0, None)])
+@pytest.mark.parametrize("S,indep,mix,after", [(1, False, 1.0, 0), (2, True, 0.35, 0), (2, False, 1.0, 6)])
 def test_gpu_graph_boundary_steps_equal_eager(S, indep, mix, after):
     """Chunk-boundary steps replayed from their own recording against the eager path: chunks of 8
     tokens, 70 steps = 9 boundaries, a ring of two chunks (its write position wraps at every
     second boundary) next to a ring of one and an unbounded layer, and head-rooms so small that
     the summary region and the append-only buffers outgrow their buffers several times (each
     growth moves the buffers, so both recordings are made again).  `after` = how many boundary
-    steps of a cache run eagerly before they are recorded (None: the class's own number, so the
-    switch happens in the middle of the run).  Tolerance as for the steps
+    steps of a cache run eagerly before they are recorded (6: the switch happens in the middle of
+    the run).  Tolerance as for the steps
     inside a chunk: 1 % of the logit scale at every step (the two paths choose the decode
     kernel's split count differently)."""
     from ksa_amd.model import HipOps
@@ -364,8 +364,7 @@ def test_gpu_graph_boundary_steps_equal_eager(S, indep, mix, after):
         _SUMMARY_INIT_CAP = 3
     ops.cache_cls = SmallHeadroom
     model = KsaQwen3ForCausalLM(cfg, w, ops)
-    if after is not None:
-        model.BOUNDARY_GRAPH_AFTER = after
+    model.BOUNDARY_GRAPH_AFTER = after
     replays = []
     inner = model._replay
     model._replay = lambda st, which, body, cache: (replays.append(which), inner(st, which, body, cache))[1]
