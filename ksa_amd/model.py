@@ -482,8 +482,20 @@ class KsaQwen3ForCausalLM:
         v = qkv[..., (Hq + Hkv) * D:].view(b, L, Hkv, D)
         return q, k, v
 
+    # A prefill whose gate | up activation would be larger than this runs its MLP over slices of the batch
+    # (at the 4B shape a 32k prompt at batch 8 has 10.8 GB and is not sliced; at batch 64 it would be 86 GB).
+    MLP_SLICE_BYTES = 16 << 30
+
     def _mlp(self, lw, x, defer=False):
         """`defer`: the result only goes to `_add_norm` (see `HipOps.linear`)."""
+        if not defer and x.dim() == 3 and x.shape[0] > 1:
+            per_seq = x.shape[1] * lw["gate_up_proj"].shape[0] * x.element_size()
+            if per_seq * x.shape[0] > self.MLP_SLICE_BYTES:
+                n = max(1, int(self.MLP_SLICE_BYTES // per_seq))
+                out = torch.empty_like(x)
+                for i in range(0, x.shape[0], n):
+                    out[i:i + n] = self._mlp(lw, x[i:i + n])
+                return out
         if defer and hasattr(self.ops, "mlp_rows"):
             out = self.ops.mlp_rows(x, lw["gate_up_proj"], lw["down_proj"])
             if out is not None:

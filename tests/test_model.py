@@ -111,6 +111,29 @@ def test_decode_matches_prefill_inside_a_chunk_S2(m):
         assert torch.allclose(dec[:, j], ref[:, 0], atol=2e-5, rtol=1e-4), t
 
 
+def test_prefill_mlp_sliced_over_the_batch():
+    """A prefill whose MLP activation exceeds `MLP_SLICE_BYTES` runs the MLP over slices of the batch: same
+    logits as in one piece, and the same logits from the decode steps that follow (host operators; rows are
+    independent, so only the library's blocking of the products may differ)."""
+    cfg = tiny_config()
+    model, _ = cpu_model(cfg, 2)
+    ids = torch.randint(0, cfg.vocab_size, (5, 21), generator=torch.Generator().manual_seed(2))
+    log0, c0 = model.prefill(ids)
+    model.MLP_SLICE_BYTES = 2 * 21 * 2 * cfg.intermediate_size * 4   # two sequences per slice (fp32 host weights)
+    seen = []
+    inner = model.ops.silu_mul
+    model.ops.silu_mul = lambda g, u=None: (seen.append(g.shape[0]), inner(g, u))[1]
+    log1, c1 = model.prefill(ids)
+    assert torch.allclose(log0, log1, atol=1e-5, rtol=1e-5)
+    assert seen and max(seen) <= 2 and sum(seen) == 5 * cfg.num_hidden_layers
+    model.ops.silu_mul = inner
+    tok = log0.argmax(-1)
+    for _ in range(4):   # the caches hold the same rows: a few decode steps across a chunk boundary agree as well
+        d0, d1 = model.decode_step(tok, c0), model.decode_step(tok, c1)
+        assert torch.allclose(d0, d1, atol=1e-5, rtol=1e-5)
+        tok = d0.argmax(-1)
+
+
 def test_generate_shapes_and_forcing():
     cfg = tiny_config()
     model, _ = cpu_model(cfg)
