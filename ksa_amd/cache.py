@@ -118,6 +118,8 @@ class Qwen3RingBufferCache:
         self.true_tokens = [0] * n
         self._total_chunks = [0] * n
         self._reorganized = False
+        self._reorg_done = set()   # layers already in the ring layout (`reorganize_layer`)
+        self._reorg_rows = None    # (text rows, summary rows, counts) of the prefill, made once
 
     # ---- queries -------------------------------------------------------------------
     def __len__(self):
@@ -228,49 +230,58 @@ class Qwen3RingBufferCache:
         """Prefill order -> ring layout for every layer.  summary_mask: bool [bsz, prefill_len]."""
         if self._reorganized:
             return
+        for layer in range(self.num_hidden_layers):
+            self.reorganize_layer(layer, summary_mask)
         self._reorganized = True
+
+    def reorganize_layer(self, layer: int, summary_mask: torch.Tensor):
+        """`reorganize_after_prefill` for one layer, for a prefill that calls it as soon as the layer's
+        attention has run: a small-window layer then gives up all but its window and its summaries at
+        once instead of holding the whole prompt's K/V until every layer has run (at the 4B shape 27 of
+        36 layers; the reference reorganises all layers at the end, :209-302)."""
+        if self._reorganized or layer in self._reorg_done:
+            return
+        self._reorg_done.add(layer)
         C, S = self.summary_chunk_size, self.summary_token_num
-        sm = summary_mask[0]
-        text_rows = torch.nonzero(~sm, as_tuple=False).flatten().to(torch.int32)
-        sum_rows = torch.nonzero(sm, as_tuple=False).flatten().to(torch.int32)
+        if self._reorg_rows is None:
+            sm = summary_mask[0]
+            self._reorg_rows = (torch.nonzero(~sm, as_tuple=False).flatten().to(torch.int32),
+                                torch.nonzero(sm, as_tuple=False).flatten().to(torch.int32))
+        text_rows, sum_rows = self._reorg_rows
         n_text, n_sum = text_rows.numel(), sum_rows.numel()
         n_complete, n_partial = divmod(n_text, C)
 
-        for layer in range(self.num_hidden_layers):
-            old_k, old_v = self.key_cache[layer], self.value_cache[layer]
-            if self.is_large_window[layer]:
-                cap = n_text + self._APPEND_HEADROOM
-                new_k, new_v = self._alloc(old_k, cap), self._alloc(old_v, cap)
-                self._move_rows(old_k, new_k, n_text, src_index=text_rows)
-                self._move_rows(old_v, new_v, n_text, src_index=text_rows)
-                self._text_len[layer] = n_text
-            else:
-                ws, scn = self.window_sizes[layer], self.sliding_chunk_nums[layer]
-                n_win = min(scn, n_complete) * C
-                cap = S + C + ws + n_sum + max(self._SUMMARY_INIT_CAP, n_sum + 256)
-                new_k, new_v = self._alloc(old_k, cap), self._alloc(old_v, cap)
-                first_win = n_complete * C - n_win
-                for old, new in ((old_k, new_k), (old_v, new_v)):
-                    # trailing partial chunk, right-aligned in the chunk region
-                    self._move_rows(old, new, n_partial, dst_start=S + C - n_partial,
-                                    src_index=text_rows[n_complete * C:])
-                    # newest complete chunks, chronological, from the ring base
-                    self._move_rows(old, new, n_win, dst_start=S + C,
-                                    src_index=text_rows[first_win:n_complete * C])
-                    self._move_rows(old, new, n_sum, dst_start=S + C + ws, src_index=sum_rows)
-                self._n_valid_window[layer] = n_win
-                self._window_write_ptr[layer] = n_win % ws
-                self._n_summaries[layer] = n_sum
-                self._chunk_buf_len[layer] = n_partial
-                self._text_len[layer] = 0
-            self.key_cache[layer], self.value_cache[layer] = new_k, new_v
-            self._capacity[layer] = cap
-
-        block = C + S
-        for layer in range(self.num_hidden_layers):
-            self.cur_chunk_sizes[layer] %= block
-            self._total_chunks[layer] = (self.true_tokens[layer] // C if self.is_large_window[layer]
-                                         else self._n_summaries[layer])
+        old_k, old_v = self.key_cache[layer], self.value_cache[layer]
+        if self.is_large_window[layer]:
+            cap = n_text + self._APPEND_HEADROOM
+            new_k, new_v = self._alloc(old_k, cap), self._alloc(old_v, cap)
+            self._move_rows(old_k, new_k, n_text, src_index=text_rows)
+            self._move_rows(old_v, new_v, n_text, src_index=text_rows)
+            self._text_len[layer] = n_text
+        else:
+            ws, scn = self.window_sizes[layer], self.sliding_chunk_nums[layer]
+            n_win = min(scn, n_complete) * C
+            cap = S + C + ws + n_sum + max(self._SUMMARY_INIT_CAP, n_sum + 256)
+            new_k, new_v = self._alloc(old_k, cap), self._alloc(old_v, cap)
+            first_win = n_complete * C - n_win
+            for old, new in ((old_k, new_k), (old_v, new_v)):
+                # trailing partial chunk, right-aligned in the chunk region
+                self._move_rows(old, new, n_partial, dst_start=S + C - n_partial,
+                                src_index=text_rows[n_complete * C:])
+                # newest complete chunks, chronological, from the ring base
+                self._move_rows(old, new, n_win, dst_start=S + C,
+                                src_index=text_rows[first_win:n_complete * C])
+                self._move_rows(old, new, n_sum, dst_start=S + C + ws, src_index=sum_rows)
+            self._n_valid_window[layer] = n_win
+            self._window_write_ptr[layer] = n_win % ws
+            self._n_summaries[layer] = n_sum
+            self._chunk_buf_len[layer] = n_partial
+            self._text_len[layer] = 0
+        self.key_cache[layer], self.value_cache[layer] = new_k, new_v
+        self._capacity[layer] = cap
+        self.cur_chunk_sizes[layer] %= C + S
+        self._total_chunks[layer] = (self.true_tokens[layer] // C if self.is_large_window[layer]
+                                     else self._n_summaries[layer])
 
     # ---- decode ----------------------------------------------------------------------
     def update_text(self, key_states: torch.Tensor, value_states: torch.Tensor, layer_idx: int):

@@ -533,6 +533,9 @@ class KsaQwen3ForCausalLM:
                                         k_out=k_slot, v_out=v_slot)
             self._blend_summary(lw, h, sum_rows, cos, sin, q, k, v)
             attn, _ = ops.summary_attn_func(q, k, v, C, S, self.scns[li], summary_pos=is_sum)
+            del q, k, v, k_slot, v_slot
+            if hasattr(cache, "reorganize_layer"):   # the layer's K/V in prompt order are not needed any more
+                cache.reorganize_layer(li, is_sum[None])
             x, h = self._add_norm(ops.linear(attn.reshape(b, L, -1), lw["o_proj"]), x, lw["post_attention_layernorm"])
             delta = self._mlp(lw, h)
         cache.reorganize_after_prefill(is_sum[None])
