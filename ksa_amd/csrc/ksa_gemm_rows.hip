@@ -497,6 +497,7 @@ extern "C" int ksa_gemm_rows(const void* x, const void* w, void* out, int M, int
         wp.M = M, wp.N = N, wp.K = K, wp.ksplit = ksplit, wp.chunks_per_split = pl.chunks_per_split;
         if (ksplit > 1) {
             if (!workspace || workspace_bytes < ksa_gemm_rows_partials_bytes(M, N, ksplit)) return KSA_ERR_WORKSPACE;
+            if (reinterpret_cast<uintptr_t>(workspace) & 15) return KSA_ERR_ALIGN;  // 16-byte stores of the sums
             wp.part = (float*)workspace;
         }
         const int rc = dtype == KSA_DTYPE_BF16 ? launch_wide<KsaBf16, false>(wp, (hipStream_t)stream)
@@ -538,6 +539,7 @@ extern "C" int ksa_gemm_rows_gate_up_silu(const void* x, const void* w, void* ou
     if (x_row_stride % 8 || (w_row_stride != kWTiled && w_row_stride % 8)) return KSA_ERR_ALIGN;
     if (w_row_stride == kWTiled && I % 16 != 0) return KSA_ERR_UNSUPPORTED;  // gate and up rows must start tiles of their own
     if (M > 16) {  // chunks of x through LDS, gate and up waves of a workgroup meet behind the walk
+        if (reinterpret_cast<uintptr_t>(out) & 7) return KSA_ERR_ALIGN;  // 8-byte stores of the activation
         WideParams wp{};
         wp.x = (const uint16_t*)x, wp.w = (const uint16_t*)w, wp.out = (uint16_t*)out;
         wp.xs = x_row_stride, wp.ws = w_row_stride, wp.os = out_row_stride;

@@ -39,8 +39,9 @@ struct KsaWeightLane {
 __device__ __forceinline__ KsaWeightLane ksa_weight_lane(const uint16_t* w, int64_t rs, int K, int64_t row0, int r,
                                                          int kq, int64_t nrows) {
     KsaWeightLane l;
-    if (rs == kWTiled) {
-        l.p = w + (row0 / 16) * (int64_t)(K / 32) * 512 + r * 32 + 8 * kq;
+    if (rs == kWTiled) {  // (a wave whose 16 rows all lie past the matrix reads the last tile: nothing of it is stored)
+        const int64_t last = (nrows - 1) / 16;
+        l.p = w + (row0 / 16 < last ? row0 / 16 : last) * (int64_t)(K / 32) * 512 + r * 32 + 8 * kq;
         l.step = 512;
     } else {
         const int64_t row = row0 + r < nrows ? row0 + r : nrows - 1;
