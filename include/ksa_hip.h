@@ -282,7 +282,8 @@ int ksa_silu_mul_partials(const float* partials, int ksplit, void* out, int rows
  * ksa_gemm_rows_splits can return are taken - slices are whole chunks, none empty - anything else is
  * KSA_ERR_INVALID.  With ksplit > 1 out may be NULL: the partial sums (fp32 [ksplit][R][N], R = M
  * rounded up to a multiple of 16) are then left in the workspace for a consumer that adds them itself
- * (ksa_add_rmsnorm_partials, ksa_silu_mul_partials, ksa_pre_attention_partials). */
+ * (ksa_add_rmsnorm_partials, ksa_silu_mul_partials, ksa_pre_attention_partials).  x and w 16-byte
+ * aligned, for M > 16 the workspace as well (KSA_ERR_ALIGN otherwise). */
 /* The streaming layout of a weight matrix.  The few-rows kernels read a weight fragment of 16 rows x 32
  * elements of K per wave instruction - in a row-major w [N, K] that is 64 bytes of each of 16 rows K elements
  * apart.  ksa_tile_weights writes the same matrix as [ceil(N / 16)][K / 32][16][32] (rows past N: zeros;
@@ -313,7 +314,8 @@ int ksa_gemm_rows(const void* x, const void* w, void* out, int M, int N, int K, 
  *   x [M, K], w [2 I, K] (gate rows, then up rows), out [M, I]; K a multiple of 32; row strides in
  *   elements (x, w: multiples of 8).  Up to 16 rows x is held in LDS whole: M (K + 8) 2 bytes beyond
  *   160 KiB are KSA_ERR_UNSUPPORTED (use ksa_gemm_rows and ksa_silu_mul then); 17 to 128 rows go
- *   through LDS in chunks (any K), half of a workgroup's waves on gate columns, half on up columns. */
+ *   through LDS in chunks (any K), half of a workgroup's waves on gate columns, half on up columns
+ *   (out 8-byte aligned then). */
 int ksa_gemm_rows_gate_up_silu(const void* x, const void* w, void* out, int M, int I, int K,
                                long long x_row_stride, long long w_row_stride, long long out_row_stride,
                                int dtype, void* stream);
